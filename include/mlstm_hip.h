@@ -1,0 +1,99 @@
+/*
+ * mlstm_hip.h -- C ABI of libmlstm_hip.so: the mLSTM hot path (TFLA chunkwise forward/backward and the
+ * fused recurrent decode step) as hand-written gfx950 HIP kernels.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer owned by the caller; the library never allocates or frees device
+ *     memory and keeps no state between calls except a thread-local error string.
+ *   - Tensors are dense row-major: q,k (B,NH,S,DHQK); v,H,dH (B,NH,S,DHHV); i,f (B,NH,S);
+ *     C (B,NH,DHQK,DHHV) fp32; n (B,NH,DHQK) fp32; m (B,NH) fp32.
+ *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it.
+ *   - Return value 0 = success; anything else = failure, message via mlstm_hip_last_error().
+ *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1.  gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp),
+ *     MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
+ *   - Supported shapes: DHQK % 64 == 0, DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the reference checkout).
+ */
+#ifndef MLSTM_HIP_H
+#define MLSTM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLSTM_F32 0
+#define MLSTM_BF16 1
+#define MLSTM_GATE_EXP 0
+#define MLSTM_GATE_SIG 1
+
+/* ABI version of the loaded library (bumped on any signature change). */
+int mlstm_hip_abi_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* mlstm_hip_last_error(void);
+
+/*
+ * Fused recurrent decode step (one token for every (b, head)).
+ * Replaces: mlstm_kernels/torch/recurrent/triton_step.py:15-127 (mlstm_recurrent_step__triton_fw) and the
+ * Triton kernel mlstm_kernels/triton/recurrent/fw_step_fused.py:19-195.
+ *   q,k (B,NH,DHQK), v (B,NH,DHHV) in dtype_qkv; i,f (B,NH) in dtype_gates; h (B,NH,DHHV) in dtype_qkv.
+ *   c_out/n_out/m_out may alias c_in/n_in/m_in (in-place update) or be distinct buffers.
+ */
+int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f,
+                   const float* c_in, const float* n_in, const float* m_in,
+                   void* h, float* c_out, float* n_out, float* m_out,
+                   int B, int NH, int DHQK, int DHHV, float eps,
+                   int dtype_qkv, int dtype_gates, void* stream);
+
+/*
+ * Bytes of caller-provided workspace the chunkwise forward needs.  With keep_for_backward != 0 the
+ * workspace additionally holds everything the backward re-uses (gate vectors, per-chunk bf16 states,
+ * per-row normalisers) and must be handed unchanged to mlstm_hip_chunkwise_bw.
+ */
+size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int keep_for_backward);
+
+/*
+ * TFLA chunkwise forward, mLSTMexp or mLSTMsig.
+ * Replaces: mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:20-136 (mlstm_chunkwise_fw: recurrent_fw_C +
+ * parallel_fw_Hintra + gate pre-pass) and .../triton_xl_chunk_siging/fw.py for gate == MLSTM_GATE_SIG.
+ *   c0,n0,m0: initial states or NULL (all three NULL together; m0 ignored for the sig gate).
+ *   H (B,NH,S,DHHV) in dtype_qkv.  n_out, m_out: optional fp32 (B,NH,S) per-row normaliser max(|den|,floor)
+ *   and stabiliser (NULL to skip).  c_last,n_last,m_last: optional fp32 last states (NULL to skip).
+ *   normalize applies to the sig gate only (0: H is the bare numerator).
+ */
+int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const void* i, const void* f,
+                           const float* c0, const float* n0, const float* m0,
+                           void* H, float* n_out, float* m_out,
+                           float* c_last, float* n_last, float* m_last,
+                           void* workspace, size_t workspace_bytes, int keep_for_backward,
+                           int B, int NH, int S, int DHQK, int DHHV, float eps,
+                           int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream);
+
+/* Bytes of scratch the chunkwise backward needs in addition to the forward workspace. */
+size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV);
+
+/*
+ * TFLA chunkwise backward (normaliser and stabilisers are constants, as in the reference).
+ * Replaces: mlstm_kernels/torch/chunkwise/triton_xl_chunk/bw.py:27-227 (mlstm_chunkwise_bw: recurrent_bw_dC,
+ * parallel_bw_dV/dK/dQ, gate-gradient post-pass) and the siging counterpart.
+ *   fw_workspace: the forward's workspace, produced with keep_for_backward != 0 for the same inputs.
+ *   dH (B,NH,S,DHHV) in dtype_qkv; dC_last optional fp32 gradient of the last C state (NULL = zero).
+ *   dQ,dK (B,NH,S,DHQK), dV (B,NH,S,DHHV) in dtype_qkv; dI,dF fp32 (B,NH,S);
+ *   dC0 optional fp32 (B,NH,DHQK,DHHV) gradient of the initial C state (NULL to skip).
+ */
+int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const void* i, const void* f,
+                           const void* dH, const float* dC_last,
+                           void* dQ, void* dK, void* dV, float* dI, float* dF, float* dC0,
+                           const void* fw_workspace, size_t fw_workspace_bytes,
+                           void* bw_workspace, size_t bw_workspace_bytes,
+                           int B, int NH, int S, int DHQK, int DHHV, float eps,
+                           int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLSTM_HIP_H */

@@ -1,0 +1,65 @@
+"""ctypes binding of libmlstm_hip.so (C ABI in include/mlstm_hip.h).  Loading fails loudly."""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmlstm_hip.so")
+_lock = threading.Lock()
+_lib = None
+
+F32, BF16 = 0, 1
+GATE_EXP, GATE_SIG = 0, 1
+ABI_VERSION = 1
+
+_vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+
+_SIGNATURES = {
+    "mlstm_hip_abi_version": (_i, []),
+    "mlstm_hip_last_error": (ctypes.c_char_p, []),
+    "mlstm_hip_step": (_i, [_vp] * 12 + [_i, _i, _i, _i, _f, _i, _i, _vp]),
+    "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 6),
+    "mlstm_hip_chunkwise_fw": (_i, [_vp] * 15 + [_sz, _i] + [_i] * 5 + [_f] + [_i] * 4 + [_vp]),
+    "mlstm_hip_chunkwise_bw_workspace_bytes": (_sz, [_i] * 5),
+    "mlstm_hip_chunkwise_bw": (_i, [_vp] * 14 + [_sz, _vp, _sz] + [_i] * 5 + [_f] + [_i] * 4 + [_vp]),
+}
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def exported_symbols() -> list[str]:
+    return sorted(_SIGNATURES)
+
+
+def get_lib() -> ctypes.CDLL:
+    """Return the loaded library; raise RuntimeError if it was not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(_LIB_PATH):
+                raise RuntimeError(
+                    f"{_LIB_PATH} not found. The HIP kernels are the only implementation of this package; "
+                    "build them with `python -m mlstm_kernels_amd.build` (needs hipcc, targets gfx950)."
+                )
+            lib = ctypes.CDLL(_LIB_PATH)
+            for name, (res, args) in _SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = res
+                fn.argtypes = args
+            if lib.mlstm_hip_abi_version() != ABI_VERSION:
+                raise RuntimeError(
+                    f"libmlstm_hip.so has ABI version {lib.mlstm_hip_abi_version()}, expected {ABI_VERSION}; rebuild it."
+                )
+            _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = get_lib().mlstm_hip_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed: {msg}")

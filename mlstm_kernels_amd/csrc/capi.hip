@@ -1,0 +1,129 @@
+// C ABI of libmlstm_hip.so (declared in include/mlstm_hip.h): argument validation, workspace carving and
+// kernel sequencing.  No device memory is allocated here and no state is kept between calls.
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/mlstm_hip.h"
+#include "kernels.h"
+
+namespace {
+thread_local char g_err[512] = "";
+int fail(const char* msg) {
+  snprintf(g_err, sizeof(g_err), "%s", msg);
+  return 1;
+}
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+    return 1;
+  }
+  return 0;
+}
+const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {
+  if (B <= 0 || NH <= 0 || S <= 0) return "B, NH and S must be positive";
+  if (DHQK <= 0 || DHHV <= 0 || DHQK % 64 != 0 || DHHV % 64 != 0) return "DHQK and DHHV must be positive multiples of 64";
+  if ((long long)B * NH > 65535) return "B*NH exceeds 65535";
+  return nullptr;
+}
+}  // namespace
+
+extern "C" {
+
+int mlstm_hip_abi_version(void) { return 1; }
+const char* mlstm_hip_last_error(void) { return g_err; }
+
+int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c_in,
+                   const float* n_in, const float* m_in, void* h, float* c_out, float* n_out, float* m_out, int B,
+                   int NH, int DHQK, int DHHV, float eps, int dtype_qkv, int dtype_gates, void* stream) {
+  if (!q || !k || !v || !i || !f || !c_in || !n_in || !m_in || !h || !c_out || !n_out || !m_out)
+    return fail("mlstm_hip_step: null pointer argument");
+  if (n_out == n_in || m_out == m_in)
+    return fail("mlstm_hip_step: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
+  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16))
+    return fail("mlstm_hip_step: unsupported dtype code");
+  const char* e = mlstm::launch_step(q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps,
+                                     dtype_qkv, dtype_gates, (hipStream_t)stream);
+  if (e) return fail(e);
+  return check_launch("mlstm_hip_step");
+}
+
+size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int keep_for_backward) {
+  (void)keep_for_backward;
+  if (check_dims(B, NH, S, DHQK, DHHV)) return 0;
+  return mlstm::carve_fw_workspace(nullptr, B, NH, S, DHQK, DHHV).bytes;
+}
+
+int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c0,
+                           const float* n0, const float* m0, void* H, float* n_out, float* m_out, float* c_last,
+                           float* n_last, float* m_last, void* workspace, size_t workspace_bytes,
+                           int keep_for_backward, int B, int NH, int S, int DHQK, int DHHV, float eps, int dtype_qkv,
+                           int dtype_gates, int gate, int normalize, void* stream) {
+  (void)keep_for_backward;
+  if (!q || !k || !v || !i || !f || !H || !workspace) return fail("mlstm_hip_chunkwise_fw: null pointer argument");
+  if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return fail(e);
+  if (dtype_qkv != MLSTM_BF16) return fail("mlstm_hip_chunkwise_fw: q/k/v must be bf16");
+  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return fail("mlstm_hip_chunkwise_fw: unsupported gate dtype");
+  if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return fail("mlstm_hip_chunkwise_fw: unknown gate code");
+  const bool has_c0 = c0 != nullptr;
+  if (has_c0 != (n0 != nullptr)) return fail("mlstm_hip_chunkwise_fw: c0 and n0 must be given together");
+  if (gate == MLSTM_GATE_EXP && has_c0 != (m0 != nullptr))
+    return fail("mlstm_hip_chunkwise_fw: initial states must be given together");
+  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(workspace, B, NH, S, DHQK, DHHV);
+  if (workspace_bytes < ws.bytes) return fail("mlstm_hip_chunkwise_fw: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  const int NC = (S + 127) / 128, BH = B * NH;
+  const int sig = gate == MLSTM_GATE_SIG;
+  if (const char* e = mlstm::launch_gates(i, f, m0, ws.g, m_last, B, NH, S, dtype_gates, sig, st)) return fail(e);
+  if (check_launch("gates")) return 1;
+
+  mlstm::ScanArgs sa;
+  memset(&sa, 0, sizeof(sa));
+  sa.X = (const uint16_t*)k;
+  sa.Y = (const uint16_t*)v;
+  sa.scale_a = ws.g.abar;
+  sa.gbar = ws.g.gbar;
+  sa.init = c0;
+  sa.states = ws.cstates;
+  sa.final_out = c_last;
+  sa.n_init = n0;
+  sa.nstates = ws.nstates;
+  sa.n_final = n_last;
+  sa.S = S; sa.NC = NC; sa.DHQK = DHQK; sa.DHHV = DHHV;
+  sa.qk_scale = 1.0f / sqrtf((float)DHQK);
+  sa.eps = eps;
+  sa.backward = 0;
+  if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/true, st)) return fail(e);
+  if (check_launch("scan_fw")) return 1;
+
+  mlstm::ParFwArgs pa;
+  memset(&pa, 0, sizeof(pa));
+  pa.Q = (const uint16_t*)q; pa.K = (const uint16_t*)k; pa.V = (const uint16_t*)v;
+  pa.g = ws.g;
+  pa.nstates = ws.nstates;
+  pa.cstates = ws.cstates;
+  pa.nrow = ws.nrow;
+  pa.H = (uint16_t*)H;
+  pa.n_out = n_out; pa.m_out = m_out;
+  pa.S = S; pa.NC = NC; pa.DHQK = DHQK; pa.DHHV = DHHV;
+  pa.qk_scale = sa.qk_scale; pa.eps = eps;
+  pa.sig_gate = sig; pa.normalize = normalize;
+  if (const char* e = mlstm::launch_par_fw(pa, BH, st)) return fail(e);
+  return check_launch("par_fw");
+}
+
+size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV) {
+  if (check_dims(B, NH, S, DHQK, DHHV)) return 0;
+  return mlstm::carve_bw_workspace(nullptr, B, NH, S, DHQK, DHHV).bytes;
+}
+
+int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const void* i, const void* f, const void* dH,
+                           const float* dC_last, void* dQ, void* dK, void* dV, float* dI, float* dF, float* dC0,
+                           const void* fw_workspace, size_t fw_workspace_bytes, void* bw_workspace,
+                           size_t bw_workspace_bytes, int B, int NH, int S, int DHQK, int DHHV, float eps,
+                           int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream) {
+  return fail("mlstm_hip_chunkwise_bw: not implemented yet");
+}
+
+}  // extern "C"

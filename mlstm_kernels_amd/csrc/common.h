@@ -1,0 +1,77 @@
+// Shared device helpers for the gfx950 mLSTM kernels: vector types, bf16 packing, MFMA wrappers,
+// LDS fragment reads (plain and transposing), wave-level scans.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mlstm {
+
+constexpr int kWave = 64;
+constexpr int kChunk = 128;  // internal chunk length L of every chunkwise kernel
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+// 8 bf16 as raw bits; convertible to the MFMA operand type without data movement
+union Frag {
+  uint4 u;
+  bf16x8 v;
+  uint16_t h[8];
+  uint32_t w[4];
+  uint2 d[2];
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bits (finite inputs; NaN stays NaN via the quiet bit)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+// D(32x32) += A(32x16) * B(16x32), bf16 operands, fp32 accumulate.
+// lane l: r = l % 32, h = l / 32.  A frag: A[r][8h..8h+7]; B frag: B[8h..8h+7][r];
+// acc[i] = D[8*(i/4) + 4h + (i%4)][r].
+__device__ __forceinline__ void mfma32(f32x16& acc, const Frag& a, const Frag& b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
+}
+
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// Transposing 64-bit LDS read.  Within each block of 16 lanes, lane i must pass the address of the 4
+// consecutive 16-bit elements T[k0 + i/4][n0 + 4*(i%4) .. +3]; it receives T[k0 .. k0+3][n0 + i].
+__device__ __forceinline__ uint2 lds_read_tr16(const void* p) {
+  s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+  union { s16x4 s; uint2 u; } c;
+  c.s = r;
+  return c.u;
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+  return x;
+}
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
+  return x;
+}
+
+__device__ __forceinline__ float log_sigmoid(float x) {
+  // log(sigmoid(x)) = min(x, 0) - log1p(exp(-|x|))
+  return fminf(x, 0.f) - log1pf(__expf(-fabsf(x)));
+}
+
+__device__ __forceinline__ float load_scalar(const void* p, size_t idx, int dtype) {
+  return dtype == 0 ? ((const float*)p)[idx] : bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+}
+
+}  // namespace mlstm

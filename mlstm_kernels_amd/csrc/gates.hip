@@ -1,0 +1,177 @@
+// Gate pre-pass of the chunkwise mLSTM kernels.
+//
+// Every stabiliser of the chunkwise formulation depends on the gate pre-activations only, never on q/k/v.
+// This pass therefore turns (i, f) into the fp32 vectors the matrix kernels consume, so that their inner
+// loops are plain scaled GEMM chains with no running-max rescaling:
+//
+//   per position t of chunk c (chunk length 128, b = inclusive within-chunk cumsum of logsig(f),
+//   it = i for the exponential gate, logsig(i) for the sigmoid gate):
+//     m_comb[t] = max(b_t + m_{c-1}, b_t + max_{j<=t}(it_j - b_j))          (0 for the sigmoid gate)
+//     u[t]      = b_t - m_comb[t]            w[t] = b_t - it_t        => D[t][j] = exp(u[t] - w[j]), j <= t
+//     bbar[t]   = exp(b_t + m_{c-1} - m_comb[t])                        (weight of the incoming state)
+//     abar[t]   = exp(sum_{u>t} logsig(f_u) + it_t - m_c)               (weight of k_t v_t^T in C_c)
+//   per chunk c:  gbar[c] = exp(g_c + m_{c-1} - m_c),  m_c = max(g_c + m_{c-1}, max_t a_t)   (m = 0 for sig)
+//
+// (formulas of mlstm_kernels/torch/chunkwise/native/fw.py:81-121,171-190 in the reference.)  Positions past
+// the sequence end inside the last chunk get logsig(f) = 0 and it = -inf, i.e. they neither decay nor feed
+// the state, so any sequence length is handled.
+//
+// One workgroup per (batch, head): phase 1 does the within-chunk scans wave-parallel, phase 2 scans the
+// (max,+) recurrence of m over chunks with one wave (the recurrence is associative), phase 3 is elementwise.
+#include "common.h"
+#include "kernels.h"
+
+namespace mlstm {
+
+constexpr int kGateThreads = 1024;
+
+template <typename Op>
+__device__ __forceinline__ float wave_incl_scan(float x, Op op, float identity) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float y = __shfl_up(x, o);
+    x = lane >= o ? op(y, x) : x;
+  }
+  (void)identity;
+  return x;
+}
+template <typename Op>
+__device__ __forceinline__ float wave_rev_incl_scan(float x, Op op) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float y = __shfl_down(x, o);
+    x = lane + o < 64 ? op(y, x) : x;
+  }
+  return x;
+}
+
+__global__ __launch_bounds__(kGateThreads) void gates_kernel(
+    const void* __restrict__ ig, const void* __restrict__ fg, const float* __restrict__ m0,
+    GateBufs gb, float* __restrict__ m_last, int S, int NC, int dtype_gates, int sig_gate) {
+  const int bh = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const size_t Sp = (size_t)NC * kChunk;
+  float* u = gb.u + bh * Sp;          // phase 1: b
+  float* wv = gb.w + bh * Sp;
+  float* abar = gb.abar + bh * Sp;    // phase 1: a
+  float* bbar = gb.bbar + bh * Sp;
+  float* mcomb = gb.mcomb + bh * Sp;  // phase 1: b + cummax(it - b)
+  float* gbar = gb.gbar + (size_t)bh * NC;  // phase 1: g
+  float* amax = gb.amax + (size_t)bh * NC;
+  float* mst = gb.mstates + (size_t)bh * (NC + 1);
+  const float NEG_INF = -__builtin_inff();
+  auto add = [](float a, float b) { return a + b; };
+  auto mx = [](float a, float b) { return fmaxf(a, b); };
+
+  // ---- phase 1: within-chunk scans, one wave per chunk, two positions per lane
+  for (int c = wave; c < NC; c += kGateThreads / kWave) {
+    const int t0 = c * kChunk + 2 * lane;
+    float lf[2], it[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int t = t0 + e;
+      if (t < S) {
+        const size_t o = (size_t)bh * S + t;
+        lf[e] = log_sigmoid(load_scalar(fg, o, dtype_gates));
+        const float iv = load_scalar(ig, o, dtype_gates);
+        it[e] = sig_gate ? log_sigmoid(iv) : iv;
+      } else {
+        lf[e] = 0.f;
+        it[e] = NEG_INF;
+      }
+    }
+    const float pair = lf[0] + lf[1];
+    const float incl = wave_incl_scan(pair, add, 0.f);
+    const float b1 = incl, b0 = (incl - pair) + lf[0];
+    const float g = __shfl(incl, 63);
+    const float rincl = wave_rev_incl_scan(pair, add);
+    const float suf1 = rincl - pair, suf0 = suf1 + lf[1];
+    const float a0 = suf0 + it[0], a1 = suf1 + it[1];
+    const float x0 = it[0] - b0, x1 = it[1] - b1;
+    const float pm = wave_incl_scan(fmaxf(x0, x1), mx, NEG_INF);
+    float pm_excl = __shfl_up(pm, 1);
+    if (lane == 0) pm_excl = NEG_INF;
+    const float cm0 = fmaxf(pm_excl, x0), cm1 = pm;
+    const float am = wave_max(fmaxf(a0, a1));
+    *(float2*)(u + t0) = make_float2(b0, b1);
+    *(float2*)(mcomb + t0) = make_float2(b0 + cm0, b1 + cm1);
+    *(float2*)(abar + t0) = make_float2(a0, a1);
+    *(float2*)(wv + t0) = make_float2(b0 - it[0], b1 - it[1]);
+    if (lane == 0) {
+      gbar[c] = g;
+      amax[c] = am;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 2: m_c = max(g_c + m_{c-1}, amax_c) over chunks; (G, A) pairs compose associatively:
+  //      (G1, A1) then (G2, A2)  ==  (G1 + G2, max(A1 + G2, A2))
+  if (wave == 0) {
+    const float m_init = (m0 != nullptr && !sig_gate) ? m0[bh] : 0.f;
+    const int R = (NC + 63) / 64;
+    const int c_lo = min(lane * R, NC), c_hi = min(c_lo + R, NC);
+    if (sig_gate) {
+      for (int c = c_lo; c < c_hi; ++c) {
+        mst[c] = 0.f;
+        gbar[c] = expf(gbar[c]);
+      }
+      if (lane == 63) mst[NC] = 0.f;
+    } else {
+      float G = 0.f, A = NEG_INF;
+      for (int c = c_lo; c < c_hi; ++c) {
+        const float gc = gbar[c];
+        A = fmaxf(A + gc, amax[c]);
+        G += gc;
+      }
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float Gp = __shfl_up(G, o), Ap = __shfl_up(A, o);
+        if (lane >= o) {
+          A = fmaxf(Ap + G, A);
+          G = Gp + G;
+        }
+      }
+      float Gex = __shfl_up(G, 1), Aex = __shfl_up(A, 1);
+      if (lane == 0) {
+        Gex = 0.f;
+        Aex = NEG_INF;
+      }
+      float m = fmaxf(m_init + Gex, Aex);
+      for (int c = c_lo; c < c_hi; ++c) {
+        const float gc = gbar[c];
+        const float mn = fmaxf(m + gc, amax[c]);
+        mst[c] = m;
+        gbar[c] = expf(gc + m - mn);
+        m = mn;
+      }
+      // the lane that owns the last chunk holds the final m
+      if (c_hi == NC && c_lo < NC) mst[NC] = m;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase 3: elementwise finalisation
+  for (size_t t = tid; t < Sp; t += kGateThreads) {
+    const int c = (int)(t / kChunk);
+    const float mp = mst[c], mn = mst[c + 1];
+    const float b = u[t], mi = mcomb[t], a = abar[t];
+    const float mc = sig_gate ? 0.f : fmaxf(b + mp, mi);
+    u[t] = b - mc;
+    bbar[t] = expf(b + mp - mc);
+    abar[t] = expf(a - mn);
+    mcomb[t] = mc;
+  }
+  if (tid == 0 && m_last != nullptr) m_last[bh] = mst[NC];
+}
+
+const char* launch_gates(const void* i, const void* f, const float* m0, const GateBufs& gb, float* m_last,
+                         int B, int NH, int S, int dtype_gates, int sig_gate, hipStream_t stream) {
+  const int NC = (S + kChunk - 1) / kChunk;
+  hipLaunchKernelGGL(gates_kernel, dim3(B * NH), dim3(kGateThreads), 0, stream, i, f, m0, gb, m_last, S, NC,
+                     dtype_gates, sig_gate);
+  return nullptr;
+}
+
+}  // namespace mlstm

@@ -1,0 +1,240 @@
+// Inter-chunk state scan of the chunkwise mLSTM, forward (C states) and backward (dC states).
+//
+//   forward :  C_c  = gbar_c * C_{c-1} + K_c^T (abar . V_c)          c = 0 .. NC-1      (and n likewise)
+//   backward:  dC_{c-1} = gbar_c * dC_c + Q_c^T (rho . dH_c)          c = NC-1 .. 0,
+//              rho_t = bbar_t / sqrt(DHQK) / (nrow_t + eps)
+//
+// (mlstm_kernels/torch/chunkwise/native/fw.py:88-121 and bw.py:67-98 in the reference.)  Both are the same
+// kernel: a (DHQK x DHHV) fp32 state tile stays in MFMA accumulators for the whole sequence; per chunk the
+// tile is first written out as bf16 operand fragments (the state *before* the update, which is what the
+// chunk-parallel kernels consume), then decayed and updated with X_c^T (rowscale . Y_c), contraction over
+// the 128 chunk positions.  Both operands have the contraction index as their slow memory dimension, so
+// both are staged row-major in LDS and fetched with the transposing 64-bit LDS read.
+//
+// The row scale is applied to Y (the narrower operand of the tile) in fp32 before rounding to bf16.  For the
+// forward the scaled rows are split into a bf16 head and a bf16 remainder (two MFMAs) so that the final
+// state keeps ~16 mantissa bits: a single bf16 rounding of abar*V leaves a relative error of about 1.5e-3
+// in C, above the 1e-3 the state is specified to.
+#include "common.h"
+#include "kernels.h"
+
+namespace mlstm {
+
+
+template <int RT, int WT, bool HILO>
+__global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanArgs a) {
+  constexpr int WC = WT / 64;
+  constexpr int NT = 64 * (RT / 64) * WC;
+  constexpr int XS = RT + 16;  // LDS row strides (elements); +16 keeps 4 consecutive rows on distinct banks
+  constexpr int YS = WT + 16;
+  constexpr int XV = 128 * RT / 8 / NT;  // 16-byte vectors per thread per chunk
+  constexpr int YV = 128 * WT / 8 / NT;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint16_t* Xs = (uint16_t*)smem_raw;
+  uint16_t* Yh = Xs + 128 * XS;
+  uint16_t* Yl = Yh + 128 * YS;
+  float* sc = (float*)(Yl + (HILO ? 128 * YS : 0));  // [128] row scale of the current chunk
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wr = wave / WC, wc = wave % WC;
+  const int r = lane & 31, h = lane >> 5;
+  const int bh = blockIdx.z;
+  const int d_tile = blockIdx.x * RT, w_tile = blockIdx.y * WT;
+  const int d_wave = d_tile + wr * 64, w_wave = w_tile + wc * 64;
+  const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
+  const size_t Sp = (size_t)NC * kChunk;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int db = 0; db < 2; ++db)
+#pragma unroll
+    for (int wb = 0; wb < 2; ++wb) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float v0 = 0.f;
+        if (a.init != nullptr) {
+          const int d = d_wave + 32 * db + 8 * (i / 4) + 4 * h + (i % 4);
+          const int w = w_wave + 32 * wb + r;
+          v0 = a.init[((size_t)bh * DHQK + d) * DHHV + w];
+        }
+        acc[db][wb][i] = v0;
+      }
+    }
+  const bool do_n = (a.nstates != nullptr) && blockIdx.y == 0 && tid < RT;
+  float nval = 0.f;
+  if (do_n && a.n_init != nullptr) nval = a.n_init[(size_t)bh * DHQK + d_tile + tid];
+
+  const uint16_t* Xg = a.X + (size_t)bh * S * DHQK + d_tile;
+  const uint16_t* Yg = a.Y + (size_t)bh * S * DHHV + w_tile;
+
+  uint4 xr[XV], yr[YV];
+  float ysc[YV];
+  auto prefetch = [&](int c) {
+#pragma unroll
+    for (int v = 0; v < XV; ++v) {
+      const int idx = tid + v * NT;
+      const int j = idx / (RT / 8), cv = idx % (RT / 8);
+      const int t = c * kChunk + j;
+      xr[v] = t < S ? *(const uint4*)(Xg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < YV; ++v) {
+      const int idx = tid + v * NT;
+      const int j = idx / (WT / 8), cv = idx % (WT / 8);
+      const int t = c * kChunk + j;
+      yr[v] = t < S ? *(const uint4*)(Yg + (size_t)t * DHHV + cv * 8) : make_uint4(0, 0, 0, 0);
+      float s = a.scale_a[bh * Sp + t];
+      if (a.backward) {
+        s *= a.qk_scale;
+        if (a.nrow != nullptr) s /= (a.nrow[bh * Sp + t] + a.eps);
+      }
+      ysc[v] = t < S ? s : 0.f;
+    }
+  };
+
+  const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
+  prefetch(c_first);
+  for (int it = 0; it < NC; ++it) {
+    const int c = c_first + it * c_step;
+    // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split)
+#pragma unroll
+    for (int v = 0; v < XV; ++v) {
+      const int idx = tid + v * NT;
+      const int j = idx / (RT / 8), cv = idx % (RT / 8);
+      *(uint4*)(Xs + j * XS + cv * 8) = xr[v];
+    }
+#pragma unroll
+    for (int v = 0; v < YV; ++v) {
+      const int idx = tid + v * NT;
+      const int j = idx / (WT / 8), cv = idx % (WT / 8);
+      const uint32_t in[4] = {yr[v].x, yr[v].y, yr[v].z, yr[v].w};
+      uint32_t hi[4], lo[4];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const float e0 = __uint_as_float(in[p] << 16) * ysc[v];
+        const float e1 = __uint_as_float(in[p] & 0xffff0000u) * ysc[v];
+        const uint16_t h0 = f32_to_bf16_bits(e0), h1 = f32_to_bf16_bits(e1);
+        hi[p] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+        if (HILO) lo[p] = pack_bf16x2(e0 - bf16_bits_to_f32(h0), e1 - bf16_bits_to_f32(h1));
+      }
+      *(uint4*)(Yh + j * YS + cv * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+      if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      if (cv == 0) sc[j] = ysc[v];
+    }
+    __syncthreads();
+    if (it + 1 < NC) prefetch(c + c_step);
+
+    // ---- emit the state before this chunk's update as bf16 operand fragments
+    {
+      const size_t ND = DHQK / 16, NW = DHHV / 32;
+      uint4* st = (uint4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
+#pragma unroll
+      for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int wb = 0; wb < 2; ++wb) {
+          const size_t W32 = (w_wave + 32 * wb) / 32, D16 = (d_wave + 32 * db) / 16;
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            uint4 f;
+            f.x = pack_bf16x2(acc[db][wb][8 * half + 0], acc[db][wb][8 * half + 1]);
+            f.y = pack_bf16x2(acc[db][wb][8 * half + 2], acc[db][wb][8 * half + 3]);
+            f.z = pack_bf16x2(acc[db][wb][8 * half + 4], acc[db][wb][8 * half + 5]);
+            f.w = pack_bf16x2(acc[db][wb][8 * half + 6], acc[db][wb][8 * half + 7]);
+            st[(W32 * ND + D16 + half) * 64 + lane] = f;
+          }
+        }
+    }
+    // ---- decay, then accumulate X^T (scale . Y) over the 128 positions of the chunk
+    const float g = a.gbar[(size_t)bh * NC + c];
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int wb = 0; wb < 2; ++wb) acc[db][wb] *= g;
+
+    const int q16 = (lane >> 4) & 1, i16 = lane & 15;
+    const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
+#pragma unroll
+    for (int js = 0; js < 8; ++js) {
+      Frag A[2], Bh[2], Bl[2];
+#pragma unroll
+      for (int db = 0; db < 2; ++db) {
+        const uint16_t* p = Xs + (16 * js + krow) * XS + (wr * 64 + 32 * db + ncol);
+        A[db].d[0] = lds_read_tr16(p);
+        A[db].d[1] = lds_read_tr16(p + 4 * XS);
+      }
+#pragma unroll
+      for (int wb = 0; wb < 2; ++wb) {
+        const int o = (16 * js + krow) * YS + (wc * 64 + 32 * wb + ncol);
+        Bh[wb].d[0] = lds_read_tr16(Yh + o);
+        Bh[wb].d[1] = lds_read_tr16(Yh + o + 4 * YS);
+        if (HILO) {
+          Bl[wb].d[0] = lds_read_tr16(Yl + o);
+          Bl[wb].d[1] = lds_read_tr16(Yl + o + 4 * YS);
+        }
+      }
+#pragma unroll
+      for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int wb = 0; wb < 2; ++wb) {
+          mfma32(acc[db][wb], A[db], Bh[wb]);
+          if (HILO) mfma32(acc[db][wb], A[db], Bl[wb]);
+        }
+    }
+    // ---- normaliser vector (forward, first column tile only): n = gbar n + sum_j abar_j k_j
+    if (do_n) {
+      a.nstates[((size_t)bh * NC + c) * DHQK + d_tile + tid] = nval;
+      float s = 0.f;
+#pragma unroll 8
+      for (int j = 0; j < 128; ++j) s += sc[j] * bf16_bits_to_f32(Xs[j * XS + tid]);
+      nval = g * nval + s;
+    }
+    __syncthreads();
+  }
+
+  if (a.final_out != nullptr) {
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+      for (int wb = 0; wb < 2; ++wb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int d = d_wave + 32 * db + 8 * (i / 4) + 4 * h + (i % 4);
+          const int w = w_wave + 32 * wb + r;
+          a.final_out[((size_t)bh * DHQK + d) * DHHV + w] = acc[db][wb][i];
+        }
+  }
+  if (do_n && a.n_final != nullptr) a.n_final[(size_t)bh * DHQK + d_tile + tid] = nval;
+}
+
+template <int RT, int WT, bool HILO>
+static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
+  constexpr int NT = 64 * (RT / 64) * (WT / 64);
+  const size_t smem = (size_t)128 * (RT + 16) * 2 + (size_t)128 * (WT + 16) * 2 * (HILO ? 2 : 1) + 128 * 4;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+      return "scan: cannot raise the dynamic LDS limit";
+    attr_set = true;
+  }
+  dim3 grid(a.DHQK / RT, a.DHHV / WT, BH);
+  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO>), grid, dim3(NT), smem, stream, a);
+  return nullptr;
+}
+
+const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream) {
+  if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "scan: DHQK and DHHV must be multiples of 64";
+  const bool r128 = a.DHQK % 128 == 0, w128 = a.DHHV % 128 == 0;
+  if (hilo) {
+    if (r128 && w128) return launch_scan_t<128, 128, true>(a, BH, stream);
+    if (r128) return launch_scan_t<128, 64, true>(a, BH, stream);
+    if (w128) return launch_scan_t<64, 128, true>(a, BH, stream);
+    return launch_scan_t<64, 64, true>(a, BH, stream);
+  }
+  if (r128 && w128) return launch_scan_t<128, 128, false>(a, BH, stream);
+  if (r128) return launch_scan_t<128, 64, false>(a, BH, stream);
+  if (w128) return launch_scan_t<64, 128, false>(a, BH, stream);
+  return launch_scan_t<64, 64, false>(a, BH, stream);
+}
+
+}  // namespace mlstm

@@ -1,0 +1,208 @@
+"""TFLA chunkwise mLSTM (forward + backward) on the HIP kernels: mLSTMexp and mLSTMsig.
+
+Mirrors the public operators of the reference,
+  mlstm_kernels/torch/chunkwise/triton_xl_chunk/fwbw.py:244-300          (``mlstm_chunkwise__xl_chunk``)
+  mlstm_kernels/torch/chunkwise/triton_xl_chunk_siging/fwbw.py:211-269   (``mlstm_siging_chunkwise__xl_chunk``)
+with the same argument names, defaults, return structure and shape rules
+(mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:42-128).  The Triton tile-size keywords are accepted
+and ignored: the HIP kernels always work on internal chunks of 128 positions, which leaves H and the last
+states unchanged because the chunkwise formulation is exact for every chunk length."""
+from __future__ import annotations
+
+import torch
+from torch.amp import custom_bwd, custom_fwd
+
+from ... import _lib
+from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu
+
+_IGNORED_TUNING_KWARGS = (
+    "chunk_size_inter", "chunk_size_intra", "siz_b_L_parallel", "siz_b_L_loop", "siz_b_DH_parallel",
+    "siz_b_DH_loop", "num_warps_intra", "num_warps_inter", "num_stages_intra", "num_stages_inter",
+    "recompute_states_in_bw",
+)
+
+
+def _is_pow2(x: int) -> bool:
+    return x > 0 and (x & (x - 1)) == 0
+
+
+def validate_xl_chunk_shapes(S: int, chunk_size: int) -> None:
+    """Shape rules of the reference's xl_chunk kernels (kernel_param_heuristics.py:74-116)."""
+    assert S % 16 == 0, "Sequence length must be divisible by 16."
+    if S < 128:
+        assert _is_pow2(S), "Sequence length must be a power of 2."
+        return
+    if chunk_size >= 64:
+        assert chunk_size % 64 == 0, "Target chunk size must be divisible by the default chunk block size 64."
+    assert S % chunk_size == 0, f"Sequence length must be divisible by the target chunk size {chunk_size}."
+
+
+def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep):
+    B, NH, S, DHQK = q.shape
+    DHHV = v.shape[-1]
+    dev = q.device
+    lib = _lib.get_lib()
+    ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, int(keep))
+    if ws_bytes == 0:
+        raise ValueError(
+            f"unsupported shape for the HIP chunkwise kernels: B={B}, NH={NH}, S={S}, DHQK={DHQK}, DHHV={DHHV} "
+            "(head dimensions must be multiples of 64, B*NH <= 65535)"
+        )
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
+    if want_last:
+        c_last = torch.empty(B, NH, DHQK, DHHV, dtype=torch.float32, device=dev)
+        n_last = torch.empty(B, NH, DHQK, dtype=torch.float32, device=dev)
+        m_last = torch.empty(B, NH, 1, dtype=torch.float32, device=dev)
+    else:
+        c_last = n_last = m_last = None
+    rc = lib.mlstm_hip_chunkwise_fw(
+        ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0),
+        ptr(H), None, None, ptr(c_last), ptr(n_last), ptr(m_last),
+        ptr(ws), ws_bytes, int(keep), B, NH, S, DHQK, DHHV, float(eps),
+        _lib.BF16, dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize),
+        current_stream_ptr(dev),
+    )
+    _lib.check(rc, "mlstm_hip_chunkwise_fw")
+    return H, c_last, n_last, m_last, ws
+
+
+def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
+    dev = require_gpu(q, k, v, i, f)
+    B, NH, S, DHQK = q.shape
+    assert k.shape == (B, NH, S, DHQK), f"k has wrong shape {tuple(k.shape)}"
+    assert v.shape[:3] == (B, NH, S), f"v has wrong shape {tuple(v.shape)}"
+    assert i.shape == (B, NH, S) and f.shape == (B, NH, S), "i and f must have shape (B, NH, S)"
+    bf = torch.bfloat16
+    qb, kb, vb = (t.to(bf).contiguous() for t in (q, k, v))
+    gate_dt = torch.bfloat16 if (i.dtype == bf and f.dtype == bf) else torch.float32
+    ib, fb = i.to(gate_dt).contiguous(), f.to(gate_dt).contiguous()
+    if c0 is not None:
+        assert n0 is not None, "Initial states must be provided together."
+        if not siging:
+            assert m0 is not None, "Initial states must be provided together."
+        c0 = c0.to(torch.float32).contiguous()
+        n0 = n0.to(torch.float32).contiguous()
+        m0 = None if (siging or m0 is None) else m0.to(torch.float32).reshape(B, NH).contiguous()
+    else:
+        n0 = m0 = None
+    return dev, qb, kb, vb, ib, fb, c0, n0, m0
+
+
+def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool):
+    class _HipChunkwiseFwBw(torch.autograd.Function):
+        @staticmethod
+        @custom_fwd(device_type="cuda", cast_inputs=autocast_kernel_dtype)
+        def forward(ctx, q, k, v, i, f, c0, n0, m0, return_last_states, eps):
+            out_dtype = q.dtype
+            dev, qb, kb, vb, ib, fb, c0f, n0f, m0f = _prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
+            needs_bw = any(ctx.needs_input_grad[:6])
+            H, c_last, n_last, m_last, ws = _fw_launch(
+                qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw
+            )
+            ctx.save_for_backward(qb, kb, vb, ib, fb, ws)
+            ctx.cfg = (eps, q.dtype, k.dtype, v.dtype, i.dtype, f.dtype,
+                       None if c0 is None else c0.dtype, n0 is not None, m0 is not None)
+            H = H if out_dtype == torch.bfloat16 else H.to(out_dtype)
+            return H, c_last, n_last, m_last
+
+        @staticmethod
+        @custom_bwd(device_type="cuda")
+        def backward(ctx, dH, dC_last, dn_last, dm_last):
+            qb, kb, vb, ib, fb, ws = ctx.saved_tensors
+            eps, qdt, kdt, vdt, idt, fdt, c0dt, has_n0, has_m0 = ctx.cfg
+            B, NH, S, DHQK = qb.shape
+            DHHV = vb.shape[-1]
+            dev = qb.device
+            lib = _lib.get_lib()
+            bw_bytes = lib.mlstm_hip_chunkwise_bw_workspace_bytes(B, NH, S, DHQK, DHHV)
+            bws = torch.empty(bw_bytes, dtype=torch.uint8, device=dev)
+            dHb = dH.to(torch.bfloat16).contiguous()
+            dCl = None if dC_last is None else dC_last.to(torch.float32).contiguous()
+            dQ, dK, dV = torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb)
+            dI = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
+            dF = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
+            dC0 = torch.empty(B, NH, DHQK, DHHV, dtype=torch.float32, device=dev) if c0dt is not None else None
+            rc = lib.mlstm_hip_chunkwise_bw(
+                ptr(qb), ptr(kb), ptr(vb), ptr(ib), ptr(fb), ptr(dHb), ptr(dCl),
+                ptr(dQ), ptr(dK), ptr(dV), ptr(dI), ptr(dF), ptr(dC0),
+                ptr(ws), ws.numel(), ptr(bws), bw_bytes, B, NH, S, DHQK, DHHV, float(eps),
+                _lib.BF16, dtype_code(ib), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize),
+                current_stream_ptr(dev),
+            )
+            _lib.check(rc, "mlstm_hip_chunkwise_bw")
+            dn0 = torch.zeros(B, NH, DHQK, dtype=torch.float32, device=dev) if has_n0 else None
+            dm0 = torch.zeros(B, NH, 1, dtype=torch.float32, device=dev) if has_m0 else None
+            return (dQ.to(qdt), dK.to(kdt), dV.to(vdt), dI.to(idt), dF.to(fdt),
+                    None if dC0 is None else dC0.to(c0dt), dn0, dm0, None, None)
+
+    return _HipChunkwiseFwBw
+
+
+_FWBW_CACHE: dict = {}
+
+
+def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool):
+    if autocast_kernel_dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise ValueError(f"Unsupported kernel dtype {autocast_kernel_dtype}.")
+    key = (autocast_kernel_dtype, siging, normalize)
+    if key not in _FWBW_CACHE:
+        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize)
+    return _FWBW_CACHE[key]
+
+
+def mlstm_chunkwise__hip_xl_chunk(
+    q: torch.Tensor,  # (B, NH, S, DHQK)
+    k: torch.Tensor,  # (B, NH, S, DHQK)
+    v: torch.Tensor,  # (B, NH, S, DHHV)
+    i: torch.Tensor,  # (B, NH, S)
+    f: torch.Tensor,  # (B, NH, S)
+    c_initial: torch.Tensor = None,  # (B, NH, DHQK, DHHV)
+    n_initial: torch.Tensor = None,  # (B, NH, DHQK)
+    m_initial: torch.Tensor = None,  # (B, NH, 1)
+    return_last_states: bool = False,
+    eps: float = 1e-6,
+    chunk_size: int = 128,
+    autocast_kernel_dtype: torch.dtype = torch.float32,
+    **tuning_kwargs,
+):
+    """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
+    ``(H, (C_last fp32 (B,NH,DHQK,DHHV), n_last fp32 (B,NH,DHQK), m_last fp32 (B,NH,1)))``.
+    The matrix kernels multiply in bf16 with fp32 accumulation whatever the input dtype."""
+    for key in tuning_kwargs:
+        if key not in _IGNORED_TUNING_KWARGS:
+            raise TypeError(f"mlstm_chunkwise__hip_xl_chunk() got an unexpected keyword argument '{key}'")
+    validate_xl_chunk_shapes(q.shape[2], chunk_size)
+    fn = _get_fwbw(autocast_kernel_dtype, False, True)
+    H, c_last, n_last, m_last = fn.apply(q, k, v, i, f, c_initial, n_initial, m_initial, return_last_states, eps)
+    if return_last_states:
+        return H, (c_last, n_last, m_last)
+    return H
+
+
+def mlstm_siging_chunkwise__hip_xl_chunk(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    i: torch.Tensor,
+    f: torch.Tensor,
+    c_initial: torch.Tensor = None,
+    n_initial: torch.Tensor = None,
+    m_initial: torch.Tensor = None,  # unused: placeholder to match the mLSTMexp interface
+    return_last_states: bool = False,
+    eps: float = 1e-6,
+    normalize: bool = True,
+    chunk_size: int = 128,
+    autocast_kernel_dtype: torch.dtype = torch.float32,
+    **tuning_kwargs,
+):
+    """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``."""
+    for key in tuning_kwargs:
+        if key not in _IGNORED_TUNING_KWARGS:
+            raise TypeError(f"mlstm_siging_chunkwise__hip_xl_chunk() got an unexpected keyword argument '{key}'")
+    validate_xl_chunk_shapes(q.shape[2], chunk_size)
+    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize))
+    H, c_last, n_last, _ = fn.apply(q, k, v, i, f, c_initial, n_initial, None, return_last_states, eps)
+    if return_last_states:
+        return H, (c_last, n_last)
+    return H

@@ -1,0 +1,133 @@
+"""Fused recurrent decode step on the HIP kernel, plus the token loop built on it.
+
+Mirrors mlstm_kernels/torch/recurrent/triton_step.py:15-158 (``mlstm_recurrent_step__triton_fw`` /
+``mlstm_recurrent_step__triton``) and mlstm_kernels/torch/recurrent/native_sequence.py:13-122 of the
+reference: same argument names, shapes, return structure and shape assertions."""
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu
+
+
+def mlstm_recurrent_step__hip_fw(
+    matC_old: torch.Tensor,  # (B, NH, DHQK, DHHV)
+    vecN_old: torch.Tensor,  # (B, NH, DHQK)
+    scaM_old: torch.Tensor,  # (B, NH, 1)
+    vecQ: torch.Tensor,  # (B, NH, DHQK)
+    vecK: torch.Tensor,  # (B, NH, DHQK)
+    vecV: torch.Tensor,  # (B, NH, DHHV)
+    scaI: torch.Tensor,  # (B, NH, 1)
+    scaF: torch.Tensor,  # (B, NH, 1)
+    matC_new: torch.Tensor = None,
+    vecN_new: torch.Tensor = None,
+    scaM_new: torch.Tensor = None,
+    qk_scale: float = None,
+    eps: float = 1e-6,
+    dtype_state: torch.dtype = torch.float32,
+    **kwargs,
+):
+    """One step.  ``matC_new`` may be ``matC_old`` itself (in-place state update, the step then moves the
+    state through HBM exactly once each way); ``vecN_new``/``scaM_new`` must be distinct buffers."""
+    B, NH, DHQK = vecQ.shape
+    DHHV = vecV.shape[-1]
+    assert vecQ.shape == vecK.shape, "q and k must have the same shape"
+    assert matC_old.shape == (B, NH, DHQK, DHHV), f"matC_old has wrong shape, got {matC_old.shape}"
+    assert vecN_old.shape == (B, NH, DHQK), f"vecN_old has wrong shape, got {vecN_old.shape}"
+    assert scaM_old.shape == (B, NH, 1), f"scaM_old has wrong shape, got {scaM_old.shape}"
+    assert scaI.shape == (B, NH, 1), f"scaI has wrong shape, got {scaI.shape}"
+    assert scaF.shape == (B, NH, 1), f"scaF has wrong shape, got {scaF.shape}"
+    if qk_scale is not None and abs(qk_scale - DHQK ** -0.5) > 1e-12:
+        raise NotImplementedError("the HIP step kernel uses qk_scale = DHQK**-0.5")
+    if dtype_state != torch.float32:
+        raise NotImplementedError("the HIP step kernel keeps the recurrent state in float32")
+    dev = require_gpu(vecQ, vecK, vecV, scaI, scaF, matC_old, vecN_old, scaM_old)
+    q, k, v = vecQ.contiguous(), vecK.contiguous(), vecV.to(vecQ.dtype).contiguous()
+    if k.dtype != q.dtype:
+        k = k.to(q.dtype)
+    i, f = scaI.contiguous(), scaF.to(scaI.dtype).contiguous()
+    c_old = matC_old.to(torch.float32).contiguous()
+    n_old = vecN_old.to(torch.float32).contiguous()
+    m_old = scaM_old.to(torch.float32).contiguous()
+    if matC_new is None:
+        assert vecN_new is None and scaM_new is None, "Initial states must be provided together."
+        matC_new = torch.empty_like(c_old)
+        vecN_new = torch.empty_like(n_old)
+        scaM_new = torch.empty_like(m_old)
+    else:
+        assert vecN_new is not None and scaM_new is not None, "Initial states must be provided together."
+        for t in (matC_new, vecN_new, scaM_new):
+            assert t.dtype == torch.float32 and t.is_contiguous(), "state outputs must be contiguous float32"
+    h = torch.empty_like(v)
+    lib = _lib.get_lib()
+    rc = lib.mlstm_hip_step(
+        ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c_old), ptr(n_old), ptr(m_old),
+        ptr(h), ptr(matC_new), ptr(vecN_new), ptr(scaM_new),
+        B, NH, DHQK, DHHV, float(eps), dtype_code(q), dtype_code(i), current_stream_ptr(dev),
+    )
+    _lib.check(rc, "mlstm_hip_step")
+    return h, (matC_new, vecN_new, scaM_new)
+
+
+def mlstm_recurrent_step__hip(
+    q: torch.Tensor,  # (B, NH, DHQK)
+    k: torch.Tensor,  # (B, NH, DHQK)
+    v: torch.Tensor,  # (B, NH, DHHV)
+    i: torch.Tensor,  # (B, NH, 1)
+    f: torch.Tensor,  # (B, NH, 1)
+    c: torch.Tensor,  # (B, NH, DHQK, DHHV)
+    n: torch.Tensor,  # (B, NH, DHQK)
+    m: torch.Tensor,  # (B, NH, 1)
+    eps: float = 1e-6,
+    dtype_state: torch.dtype = torch.float32,
+    **kwargs,
+):
+    """Single mLSTM step: returns ``h (B,NH,DHHV)`` in q's dtype and ``(C', n', m')`` in float32."""
+    return mlstm_recurrent_step__hip_fw(
+        matC_old=c, vecN_old=n, scaM_old=m, vecQ=q, vecK=k, vecV=v, scaI=i, scaF=f,
+        eps=eps, dtype_state=dtype_state, **kwargs,
+    )
+
+
+def mlstm_recurrent_sequence__hip(
+    q: torch.Tensor,  # (B, NH, S, DHQK)
+    k: torch.Tensor,
+    v: torch.Tensor,  # (B, NH, S, DHHV)
+    i: torch.Tensor,  # (B, NH, S)
+    f: torch.Tensor,
+    c_initial: torch.Tensor = None,
+    n_initial: torch.Tensor = None,
+    m_initial: torch.Tensor = None,
+    return_last_states: bool = False,
+    eps: float = 1e-6,
+    dtype_state: torch.dtype = torch.float32,
+    **kwargs,
+):
+    """Token loop over the HIP step (used for the short remainder of a prefill).  The state is updated in
+    place in one C buffer; n and m ping-pong between two small buffers."""
+    B, NH, S, DHQK = q.shape
+    DHHV = v.shape[-1]
+    dev = require_gpu(q, k, v, i, f)
+    if c_initial is not None:
+        assert n_initial is not None and m_initial is not None, "Initial states must be provided together."
+        c = c_initial.to(torch.float32).clone()
+        n = n_initial.to(torch.float32).clone()
+        m = m_initial.to(torch.float32).clone().reshape(B, NH, 1)
+    else:
+        c = torch.zeros(B, NH, DHQK, DHHV, dtype=torch.float32, device=dev)
+        n = torch.zeros(B, NH, DHQK, dtype=torch.float32, device=dev)
+        m = torch.zeros(B, NH, 1, dtype=torch.float32, device=dev)
+    n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
+    hs = []
+    for t in range(S):
+        h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(
+            c, n, m, q[:, :, t], k[:, :, t], v[:, :, t], i[:, :, t, None], f[:, :, t, None],
+            matC_new=c, vecN_new=n_alt, scaM_new=m_alt, eps=eps, dtype_state=dtype_state,
+        )
+        n_alt, m_alt, n, m = n, m, n_new, m_new
+        hs.append(h)
+    H = torch.stack(hs, dim=-2)
+    if return_last_states:
+        return H, (c, n, m)
+    return H
