@@ -97,20 +97,21 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/true, st)) return fail(e);
   if (check_launch("scan_fw")) return 1;
 
-  mlstm::ParFwArgs pa;
+  mlstm::ParHvArgs pa;
   memset(&pa, 0, sizeof(pa));
   pa.Q = (const uint16_t*)q; pa.K = (const uint16_t*)k; pa.V = (const uint16_t*)v;
   pa.g = ws.g;
   pa.nstates = ws.nstates;
-  pa.cstates = ws.cstates;
-  pa.nrow = ws.nrow;
-  pa.H = (uint16_t*)H;
+  pa.states = ws.cstates;
+  pa.nrow_out = ws.nrow;
+  pa.Out = (uint16_t*)H;
   pa.n_out = n_out; pa.m_out = m_out;
   pa.S = S; pa.NC = NC; pa.DHQK = DHQK; pa.DHHV = DHHV;
   pa.qk_scale = sa.qk_scale; pa.eps = eps;
-  pa.sig_gate = sig; pa.normalize = normalize;
-  if (const char* e = mlstm::launch_par_fw(pa, BH, st)) return fail(e);
-  return check_launch("par_fw");
+  pa.sig_gate = sig;
+  pa.use_nrow = !(sig && !normalize);
+  if (const char* e = mlstm::launch_par_hv(pa, BH, /*is_dv=*/false, st)) return fail(e);
+  return check_launch("par_hv forward");
 }
 
 size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV) {
@@ -123,7 +124,78 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
                            const void* fw_workspace, size_t fw_workspace_bytes, void* bw_workspace,
                            size_t bw_workspace_bytes, int B, int NH, int S, int DHQK, int DHHV, float eps,
                            int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream) {
-  return fail("mlstm_hip_chunkwise_bw: not implemented yet");
+  if (!q || !k || !v || !i || !f || !dH || !dQ || !dK || !dV || !dI || !dF || !fw_workspace || !bw_workspace)
+    return fail("mlstm_hip_chunkwise_bw: null pointer argument");
+  if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return fail(e);
+  if (dtype_qkv != MLSTM_BF16) return fail("mlstm_hip_chunkwise_bw: q/k/v/dH must be bf16");
+  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return fail("mlstm_hip_chunkwise_bw: unsupported gate dtype");
+  if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return fail("mlstm_hip_chunkwise_bw: unknown gate code");
+  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(const_cast<void*>(fw_workspace), B, NH, S, DHQK, DHHV);
+  if (fw_workspace_bytes < ws.bytes) return fail("mlstm_hip_chunkwise_bw: forward workspace too small");
+  mlstm::BwWorkspace bws = mlstm::carve_bw_workspace(bw_workspace, B, NH, S, DHQK, DHHV);
+  if (bw_workspace_bytes < bws.bytes) return fail("mlstm_hip_chunkwise_bw: backward workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  const int NC = (S + 127) / 128, BH = B * NH;
+  const int sig = gate == MLSTM_GATE_SIG;
+  const int use_nrow = !(sig && !normalize);
+  const float qk_scale = 1.0f / sqrtf((float)DHQK);
+
+  mlstm::ScanArgs sa;
+  memset(&sa, 0, sizeof(sa));
+  sa.X = (const uint16_t*)q;
+  sa.Y = (const uint16_t*)dH;
+  sa.scale_a = ws.g.bbar;
+  sa.nrow = use_nrow ? ws.nrow : nullptr;
+  sa.gbar = ws.g.gbar;
+  sa.init = dC_last;
+  sa.states = bws.dcstates;
+  sa.final_out = dC0;
+  sa.S = S; sa.NC = NC; sa.DHQK = DHQK; sa.DHHV = DHHV;
+  sa.qk_scale = qk_scale; sa.eps = eps;
+  sa.backward = 1;
+  if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/false, st)) return fail(e);
+  if (check_launch("scan_bw")) return 1;
+
+  mlstm::ParHvArgs pv;
+  memset(&pv, 0, sizeof(pv));
+  pv.Q = (const uint16_t*)q; pv.K = (const uint16_t*)k; pv.V = (const uint16_t*)v; pv.dH = (const uint16_t*)dH;
+  pv.g = ws.g;
+  pv.states = bws.dcstates;
+  pv.nrow = ws.nrow;
+  pv.Out = (uint16_t*)dV;
+  pv.S = S; pv.NC = NC; pv.DHQK = DHQK; pv.DHHV = DHHV;
+  pv.qk_scale = qk_scale; pv.eps = eps;
+  pv.sig_gate = sig; pv.use_nrow = use_nrow;
+  if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
+  if (check_launch("par_hv dV")) return 1;
+
+  const int MT = DHQK % 256 == 0 ? 256 : (DHQK % 128 == 0 ? 128 : 64);
+  if (DHQK / MT > 1) {
+    // several head-dim tiles accumulate their row dots atomically: start from zero (qdq and kdk are adjacent)
+    const size_t n = (size_t)((char*)bws.kdk - (char*)bws.qdq) / 4 + (size_t)BH * NC * 128;
+    if (const char* e = mlstm::launch_fill_zero(bws.qdq, n, st)) return fail(e);
+  }
+  mlstm::ParQkArgs pq;
+  memset(&pq, 0, sizeof(pq));
+  pq.Q = (const uint16_t*)q; pq.K = (const uint16_t*)k; pq.V = (const uint16_t*)v; pq.dH = (const uint16_t*)dH;
+  pq.g = ws.g;
+  pq.nrow = ws.nrow;
+  pq.S = S; pq.NC = NC; pq.DHQK = DHQK; pq.DHHV = DHHV;
+  pq.qk_scale = qk_scale; pq.eps = eps;
+  pq.use_nrow = use_nrow;
+  pq.states = ws.cstates; pq.Out = (uint16_t*)dQ; pq.rowdot = bws.qdq;
+  if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/true, st)) return fail(e);
+  if (check_launch("par_qk dQ")) return 1;
+  pq.states = bws.dcstates; pq.Out = (uint16_t*)dK; pq.rowdot = bws.kdk;
+  if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/false, st)) return fail(e);
+  if (check_launch("par_qk dK")) return 1;
+
+  mlstm::GateGradArgs ga;
+  memset(&ga, 0, sizeof(ga));
+  ga.i = i; ga.f = f; ga.qdq = bws.qdq; ga.kdk = bws.kdk; ga.dI = dI; ga.dF = dF;
+  ga.S = S; ga.NC = NC; ga.dtype_gates = dtype_gates; ga.sig_gate = sig;
+  if (const char* e = mlstm::launch_gate_grads(ga, BH, st)) return fail(e);
+  return check_launch("gate_grads");
 }
 
 }  // extern "C"

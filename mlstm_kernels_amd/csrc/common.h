@@ -67,11 +67,23 @@ __device__ __forceinline__ float wave_max(float x) {
 
 __device__ __forceinline__ float log_sigmoid(float x) {
   // log(sigmoid(x)) = min(x, 0) - log1p(exp(-|x|))
-  return fminf(x, 0.f) - log1pf(__expf(-fabsf(x)));
+  return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
 __device__ __forceinline__ float load_scalar(const void* p, size_t idx, int dtype) {
   return dtype == 0 ? ((const float*)p)[idx] : bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+}
+
+// LDS write of one 16-byte global vector (8 consecutive head-dim entries) in the fragment order used for
+// every contraction over DHQK: inside each group of 16, entry 8a + 4h + c is stored at 8h + 4a + c.
+__device__ __forceinline__ void store_perm16(uint16_t* row, int cv, uint4 v) {
+  const int s16 = (cv >> 1) * 16, a = cv & 1;
+  *(uint2*)(row + s16 + 4 * a) = make_uint2(v.x, v.y);
+  *(uint2*)(row + s16 + 8 + 4 * a) = make_uint2(v.z, v.w);
+}
+__device__ __forceinline__ int perm16(int d) {  // position of head-dim entry d in fragment order
+  const int s16 = d & ~15, a = (d >> 3) & 1, hh = (d >> 2) & 1, c = d & 3;
+  return s16 + 8 * hh + 4 * a + c;
 }
 
 }  // namespace mlstm

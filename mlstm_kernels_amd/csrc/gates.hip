@@ -174,4 +174,55 @@ const char* launch_gates(const void* i, const void* f, const float* m0, const Ga
   return nullptr;
 }
 
+// Gate gradients (mlstm_kernels/torch/chunkwise/native/bw.py:320-326 and
+// mlstm_kernels/torch/chunkwise/triton_xl_chunk_siging/chunkwise_gates.py:72-100 in the reference):
+//   dF[t] = sigmoid(-f_t) * sum_{u >= t} (q_u.dQ_u - k_u.dK_u)     (suffix sum over the WHOLE sequence)
+//   dI[t] = k_t.dK_t   (times sigmoid(-i_t) for the sigmoid input gate)
+// One workgroup per (batch, head); every thread owns a contiguous strip, strips are combined by a
+// reverse scan over lanes and waves.
+__global__ __launch_bounds__(kGateThreads) void gate_grads_kernel(GateGradArgs a) {
+  __shared__ float wtot[kGateThreads / kWave];
+  const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int S = a.S;
+  const size_t Sp = (size_t)a.NC * kChunk;
+  const float* qdq = a.qdq + bh * Sp;
+  const float* kdk = a.kdk + bh * Sp;
+  const int R = (S + kGateThreads - 1) / kGateThreads;
+  const int lo = min(tid * R, S), hi = min(lo + R, S);
+  float tot = 0.f;
+  for (int t = lo; t < hi; ++t) tot += qdq[t] - kdk[t];
+  auto add = [](float x, float y) { return x + y; };
+  const float rincl = wave_rev_incl_scan(tot, add);       // sum over lanes >= lane
+  if (lane == 0) wtot[wave] = rincl;
+  __syncthreads();
+  float after = rincl - tot;                              // strips of higher lanes in this wave
+  for (int w = wave + 1; w < kGateThreads / kWave; ++w) after += wtot[w];
+  float run = after;
+  for (int t = hi - 1; t >= lo; --t) {
+    const size_t o = (size_t)bh * S + t;
+    const float kd = kdk[t];
+    run += qdq[t] - kd;
+    const float fv = load_scalar(a.f, o, a.dtype_gates);
+    a.dF[o] = run * (1.f / (1.f + expf(fv)));            // sigmoid(-f)
+    float di = kd;
+    if (a.sig_gate) di *= 1.f / (1.f + expf(load_scalar(a.i, o, a.dtype_gates)));
+    a.dI[o] = di;
+  }
+}
+
+__global__ void fill_zero_kernel(float* p, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream) {
+  hipLaunchKernelGGL(gate_grads_kernel, dim3(BH), dim3(kGateThreads), 0, stream, a);
+  return nullptr;
+}
+
+const char* launch_fill_zero(float* p, size_t n, hipStream_t stream) {
+  const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks > 0 ? blocks : 1), dim3(256), 0, stream, p, n);
+  return nullptr;
+}
+
 }  // namespace mlstm

@@ -26,18 +26,39 @@ struct ScanArgs {
   int backward;
 };
 
-struct ParFwArgs {
-  const uint16_t *Q, *K, *V;
+struct ParHvArgs {
+  const uint16_t *Q, *K, *V, *dH;  // forward uses Q,K,V; dV uses Q,K,dH
   GateBufs g;
-  const float* nstates;
-  const uint16_t* cstates;
-  float* nrow;      // workspace [BH][Sp]
-  uint16_t* H;      // (B,NH,S,DHHV) bf16
-  float* n_out;     // optional (B,NH,S)
-  float* m_out;     // optional (B,NH,S)
+  const float* nstates;     // forward: n before each chunk
+  const uint16_t* states;   // forward: C states; dV: dC states
+  const float* nrow;        // dV: row normaliser (input)
+  float* nrow_out;          // forward: row normaliser (output, workspace [BH][Sp])
+  uint16_t* Out;            // (B,NH,S,DHHV) bf16: H or dV
+  float* n_out;             // forward, optional (B,NH,S)
+  float* m_out;             // forward, optional (B,NH,S)
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
-  int sig_gate, normalize;
+  int sig_gate;
+  int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant
+};
+
+struct ParQkArgs {
+  const uint16_t *Q, *K, *V, *dH;
+  GateBufs g;
+  const uint16_t* states;   // dQ: C states; dK: dC states
+  const float* nrow;
+  uint16_t* Out;            // (B,NH,S,DHQK) bf16: dQ or dK
+  float* rowdot;            // [BH][Sp]: sum_d q*dQ (dQ) or sum_d k*dK (dK)
+  int S, NC, DHQK, DHHV;
+  float qk_scale, eps;
+  int use_nrow;
+};
+
+struct GateGradArgs {
+  const void *i, *f;        // gate pre-activations (B,NH,S)
+  const float *qdq, *kdk;   // [BH][Sp]
+  float *dI, *dF;           // (B,NH,S) fp32
+  int S, NC, dtype_gates, sig_gate;
 };
 
 const char* launch_step(const void* q, const void* k, const void* v, const void* i, const void* f,
@@ -47,6 +68,9 @@ const char* launch_step(const void* q, const void* k, const void* v, const void*
 const char* launch_gates(const void* i, const void* f, const float* m0, const GateBufs& gb, float* m_last,
                          int B, int NH, int S, int dtype_gates, int sig_gate, hipStream_t stream);
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream);
-const char* launch_par_fw(const ParFwArgs& a, int BH, hipStream_t stream);
+const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream);
+const char* launch_par_qk(const ParQkArgs& a, int BH, bool is_dq, hipStream_t stream);
+const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream);
+const char* launch_fill_zero(float* p, size_t n, hipStream_t stream);
 
 }  // namespace mlstm

@@ -34,7 +34,8 @@ struct FwWorkspace {
 
 struct BwWorkspace {
   uint16_t* dcstates;  // same fragment layout as cstates; index c = gradient of the state after chunk c
-  float* fdot;         // fp32 [B*NH][NC*128]: sum_d (q*dQ - k*dK) per position
+  float* qdq;          // fp32 [B*NH][NC*128]: sum_d q*dQ per position
+  float* kdk;          // fp32 [B*NH][NC*128]: sum_d k*dK per position
   size_t bytes;
 };
 
@@ -76,7 +77,8 @@ inline BwWorkspace carve_bw_workspace(void* base, int B, int NH, int S, int DHQK
   };
   BwWorkspace w;
   w.dcstates = (uint16_t*)take(BH * NC * (size_t)DHQK * DHHV * 2);
-  w.fdot = (float*)take(BH * Sp * 4);
+  w.qdq = (float*)take(BH * Sp * 4);
+  w.kdk = (float*)take(BH * Sp * 4);
   w.bytes = off;
   return w;
 }
