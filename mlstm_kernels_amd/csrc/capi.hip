@@ -87,9 +87,18 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   sa.init = c0;
   sa.states = ws.cstates;
   sa.final_out = c_last;
+  const bool track_n = !(sig && !normalize);  // the un-normalised sigmoid-gate variant leaves n untouched
   sa.n_init = n0;
-  sa.nstates = ws.nstates;
-  sa.n_final = n_last;
+  sa.nstates = track_n ? ws.nstates : nullptr;
+  sa.n_final = track_n ? n_last : nullptr;
+  if (!track_n && n_last != nullptr) {
+    if (n0 != nullptr) {
+      if (hipMemcpyAsync(n_last, n0, (size_t)BH * DHQK * sizeof(float), hipMemcpyDeviceToDevice, st) != hipSuccess)
+        return fail("mlstm_hip_chunkwise_fw: copying n0 to n_last failed");
+    } else if (const char* e = mlstm::launch_fill_zero(n_last, (size_t)BH * DHQK, st)) {
+      return fail(e);
+    }
+  }
   sa.S = S; sa.NC = NC; sa.DHQK = DHQK; sa.DHHV = DHHV;
   sa.qk_scale = 1.0f / sqrtf((float)DHQK);
   sa.eps = eps;

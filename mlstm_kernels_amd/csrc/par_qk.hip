@@ -218,8 +218,47 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
   }
   __syncthreads();
 
-  // ---- epilogue: round, transpose through LDS, coalesced store, row dots with the matching input rows
+  // ---- epilogue part 1: row dots  sum_d x[n][d] * Out[n][d]  from the fp32 accumulators (x = q for dQ, k for dK).
+  // They feed a suffix sum over the whole sequence (dF), where the rounding noise of bf16 outputs would add up
+  // like a random walk; the matching x rows are staged in LDS so every lane can read its own row.
   uint16_t* Os = Cf;
+  {
+    const uint16_t* Rg = (IS_DQ ? a.Q : a.K) + (size_t)bh * S * DHQK + d_tile;
+    constexpr int vec_per_row = MT / 8;
+    for (int idx = tid; idx < 128 * vec_per_row; idx += 256) {
+      const int j = idx / vec_per_row, cv = idx % vec_per_row;
+      const int t = t_base + j;
+      *(uint4*)(Os + j * OS + cv * 8) = t < S ? *(const uint4*)(Rg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
+    }
+  }
+  __syncthreads();
+  float* red = uu;  // [2][128]: uu/ww are dead after the gating step
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int n = 64 * ni + 32 * nb + r;
+    float part = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int d0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
+        const uint2 xv = *(const uint2*)(Os + n * OS + d0);
+        part += acc[mb][nb][4 * g4 + 0] * __uint_as_float(xv.x << 16);
+        part += acc[mb][nb][4 * g4 + 1] * __uint_as_float(xv.x & 0xffff0000u);
+        part += acc[mb][nb][4 * g4 + 2] * __uint_as_float(xv.y << 16);
+        part += acc[mb][nb][4 * g4 + 3] * __uint_as_float(xv.y & 0xffff0000u);
+      }
+    part += __shfl_xor(part, 32);
+    if (h == 0) red[mi * 128 + n] = part;
+  }
+  __syncthreads();
+  if (tid < 128) {
+    const float dot = red[tid] + red[128 + tid];
+    if (gridDim.x == 1) a.rowdot[gofs + tid] = dot;
+    else atomicAdd(a.rowdot + gofs + tid, dot);
+  }
+
+  // ---- epilogue part 2: round, transpose through LDS, coalesced store
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
     const int n = 64 * ni + 32 * nb + r;
@@ -235,29 +274,11 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
   __syncthreads();
   {
     uint16_t* Og = a.Out + (size_t)bh * S * DHQK + d_tile;
-    const uint16_t* Rg = (IS_DQ ? a.Q : a.K) + (size_t)bh * S * DHQK + d_tile;
-    constexpr int vec_per_row = MT / 8;            // 8, 16 or 32 lanes share a row
+    constexpr int vec_per_row = MT / 8;
     for (int idx = tid; idx < 128 * vec_per_row; idx += 256) {
       const int j = idx / vec_per_row, cv = idx % vec_per_row;
       const int t = t_base + j;
-      float dot = 0.f;
-      if (t < S) {
-        const uint4 ov = *(const uint4*)(Os + j * OS + cv * 8);
-        *(uint4*)(Og + (size_t)t * DHQK + cv * 8) = ov;
-        const uint4 rv = *(const uint4*)(Rg + (size_t)t * DHQK + cv * 8);
-        const uint32_t o4[4] = {ov.x, ov.y, ov.z, ov.w}, r4[4] = {rv.x, rv.y, rv.z, rv.w};
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          dot += __uint_as_float(o4[p] << 16) * __uint_as_float(r4[p] << 16);
-          dot += __uint_as_float(o4[p] & 0xffff0000u) * __uint_as_float(r4[p] & 0xffff0000u);
-        }
-      }
-#pragma unroll
-      for (int o = vec_per_row / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
-      if (cv == 0) {
-        if (gridDim.x == 1) a.rowdot[gofs + j] = dot;
-        else atomicAdd(a.rowdot + gofs + j, dot);
-      }
+      if (t < S) *(uint4*)(Og + (size_t)t * DHQK + cv * 8) = *(const uint4*)(Os + j * OS + cv * 8);
     }
   }
 }

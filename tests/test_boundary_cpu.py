@@ -1,0 +1,167 @@
+"""CPU-side checks of the operator boundary: registries, config validation, sequence-length adapters (driven
+with the oracle kernels registered under their reference names), the C-ABI library's exported symbols, and
+the absence of any CPU fallback behind the 'hip' names."""
+import os
+import re
+
+import pytest
+import torch
+
+import oracle as O
+from helpers import make_qkvif
+from mlstm_kernels_amd import _lib
+from mlstm_kernels_amd.torch import (
+    get_available_mlstm_kernels,
+    get_available_mlstm_sequence_kernels,
+    get_available_mlstm_step_kernels,
+    get_mlstm_kernel,
+    get_mlstm_sequence_kernel,
+    get_mlstm_step_kernel,
+    register_mlstm_kernel,
+    register_mlstm_sequence_kernel,
+    register_mlstm_step_kernel,
+)
+from mlstm_kernels_amd.torch.backend_module import mLSTMBackend, mLSTMBackendConfig
+from mlstm_kernels_amd.torch.chunkwise.hip_xl_chunk import validate_xl_chunk_shapes
+from mlstm_kernels_amd.torch.kernel_wrappers import wrap_chunkwise__arbitrary_sequence_length, wrap_chunkwise__pad_zeros
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _register_oracle_kernels():
+    # tests may use the oracle; the package itself never imports it
+    register_mlstm_kernel("chunkwise--native_custbw", O.mlstm_chunkwise__native_custbw)
+    register_mlstm_kernel("chunkwise--native_autograd", O.mlstm_chunkwise__native_autograd)
+    register_mlstm_step_kernel("native", O.mlstm_recurrent_step__native)
+    register_mlstm_sequence_kernel("native_sequence__native", O.mlstm_recurrent_sequence__native_fw)
+
+
+def test_registry_names_and_errors():
+    assert {"chunkwise--hip_xl_chunk", "chunkwise--hip_xl_chunk_siging"} <= set(get_available_mlstm_kernels())
+    assert "hip" in get_available_mlstm_step_kernels()
+    assert "native_sequence__hip" in get_available_mlstm_sequence_kernels()
+    assert callable(get_mlstm_kernel("chunkwise--hip_xl_chunk"))
+    assert callable(get_mlstm_step_kernel("hip"))
+    assert callable(get_mlstm_sequence_kernel("native_sequence__hip"))
+    with pytest.raises(ValueError):
+        get_mlstm_kernel("chunkwise--does_not_exist")
+    with pytest.raises(ValueError):
+        get_mlstm_kernel("nomodule--hip_xl_chunk")
+    with pytest.raises(ValueError):
+        get_mlstm_step_kernel("triton")
+    with pytest.raises(ValueError):
+        get_mlstm_sequence_kernel("nope")
+
+
+def test_config_defaults_and_validation():
+    cfg = mLSTMBackendConfig()
+    assert (cfg.chunk_size, cfg.return_last_states, cfg.autocast_kernel_dtype, cfg.eps) == (64, True, "bfloat16", 1e-6)
+    assert (cfg.inference_state_dtype, cfg.normalize_siging, cfg.mode) == ("float32", True, "train")
+    with pytest.raises(ValueError):
+        mLSTMBackendConfig(mode="train_with_padding", return_last_states=True)
+    with pytest.raises(ValueError):
+        mLSTMBackendConfig(chunkwise_kernel="parallel--native_custbw", return_last_states=True)
+    mLSTMBackendConfig(mode="train_with_padding", return_last_states=False)
+
+
+def test_shape_rules_of_the_xl_chunk_operator():
+    validate_xl_chunk_shapes(256, 128)
+    validate_xl_chunk_shapes(64, 128)   # short power-of-two sequences are one chunk
+    validate_xl_chunk_shapes(16, 64)
+    with pytest.raises(AssertionError):
+        validate_xl_chunk_shapes(250, 128)      # not a multiple of 16
+    with pytest.raises(AssertionError):
+        validate_xl_chunk_shapes(48, 64)        # < 128 and not a power of two
+    with pytest.raises(AssertionError):
+        validate_xl_chunk_shapes(384, 256)      # not divisible by the chunk size
+
+
+def test_hip_kernels_have_no_cpu_fallback():
+    q, k, v, i, f = make_qkvif(1, 1, 128, 64, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        get_mlstm_kernel("chunkwise--hip_xl_chunk")(q, k, v, i, f)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        get_mlstm_step_kernel("hip")(q[:, :, 0], k[:, :, 0], v[:, :, 0], i[:, :, :1], f[:, :, :1],
+                                     torch.zeros(1, 1, 64, 64), torch.zeros(1, 1, 64), torch.zeros(1, 1, 1))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "mlstm_hip.h")).read()
+    declared = sorted(set(re.findall(r"\b(mlstm_hip_\w+)\s*\(", header)))
+    assert declared, "no declarations found in include/mlstm_hip.h"
+    assert declared == _lib.exported_symbols(), "ctypes signature table and header disagree"
+    if not os.path.exists(_lib.lib_path()):
+        pytest.skip("libmlstm_hip.so not built (run `python -m mlstm_kernels_amd.build`)")
+    lib = _lib.get_lib()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported by the library"
+    assert lib.mlstm_hip_abi_version() == _lib.ABI_VERSION
+    # size queries and argument validation work without a GPU (no kernel is launched)
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 64, 128, 1) > 0
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 60, 128, 1) == 0
+    assert lib.mlstm_hip_chunkwise_bw_workspace_bytes(1, 2, 256, 64, 128) > 0
+    rc = lib.mlstm_hip_step(None, None, None, None, None, None, None, None, None, None, None, None,
+                            1, 1, 64, 64, 1e-6, 1, 0, None)
+    assert rc != 0 and b"null pointer" in lib.mlstm_hip_last_error()
+
+
+# ------------------------------------------------------------------ BASELINE config 1: CPU plumbing check
+def test_backend_module_train_mode_cpu_plumbing():
+    # B=1, NH=4, S=256, DHQK=64, DHHV=64, chunk_size=64, fp32, zero initial states, return_last_states=True
+    q, k, v, i, f = make_qkvif(1, 4, 256, 64, 64, seed=0, dtype=torch.float32)
+    backend = mLSTMBackend(mLSTMBackendConfig(chunkwise_kernel="chunkwise--native_custbw", sequence_kernel="native_sequence__native",
+                                              step_kernel="native", chunk_size=64, autocast_kernel_dtype="float32"))
+    H, (C, n, m) = backend(q, k, v, i, f)
+    assert H.shape == (1, 4, 256, 64) and H.dtype == q.dtype
+    assert C.shape == (1, 4, 64, 64) and n.shape == (1, 4, 64) and m.shape == (1, 4, 1)
+    H_par, _, _ = O.parallel_stablef_fw(q.double(), k.double(), v.double(), i.double(), f.double())
+    H_rec, (C_r, n_r, m_r) = O.recurrent_sequence(q.double(), k.double(), v.double(), i.double(), f.double())
+    torch.testing.assert_close(H.double(), H_par, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(H.double(), H_rec, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(C.double(), C_r, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(m.double(), m_r, rtol=1e-5, atol=1e-5)
+    assert backend(q, k, v, i, f, return_last_states=False).shape == H.shape
+
+
+@pytest.mark.parametrize("S", [1, 7, 65, 93, 500])
+def test_arbitrary_sequence_length_wrapper(S):
+    q, k, v, i, f = make_qkvif(1, 2, S, 32, 32, seed=S, dtype=torch.float64)
+    i, f = i.double(), f.double()
+    H, (C, n, m) = wrap_chunkwise__arbitrary_sequence_length(
+        mlstm_chunkwise_kernel=O.mlstm_chunkwise__native_custbw,
+        mlstm_sequence_kernel=lambda **kw: O.mlstm_recurrent_sequence__native_fw(dtype_state=torch.float64, **kw),
+        mlstm_step_kernel=lambda **kw: O.mlstm_recurrent_step__native(dtype_state=torch.float64, **kw),
+        q=q, k=k, v=v, f=f, i=i, chunk_size=64, dtype_state=torch.float64)
+    H_ref, (C_r, n_r, m_r) = O.recurrent_sequence(q, k, v, i, f)
+    torch.testing.assert_close(H, H_ref, rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(C, C_r, rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(n, n_r, rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(m, m_r, rtol=1e-9, atol=1e-9)
+
+
+def test_backend_inference_mode_threads_states():
+    q, k, v, i, f = make_qkvif(1, 2, 100, 32, 32, seed=3, dtype=torch.float32)
+    backend = mLSTMBackend(mLSTMBackendConfig(chunkwise_kernel="chunkwise--native_custbw", sequence_kernel="native_sequence__native",
+                                              step_kernel="native", chunk_size=32, mode="inference", autocast_kernel_dtype="float32"))
+    H, st = backend(q, k, v, i, f)
+    H1, st1 = backend(q[:, :, :63], k[:, :, :63], v[:, :, :63], i[:, :, :63], f[:, :, :63])
+    outs = [H1]
+    for t in range(63, 100):   # generation: one token at a time through the step kernel
+        h, st1 = backend(q[:, :, t:t + 1], k[:, :, t:t + 1], v[:, :, t:t + 1], i[:, :, t:t + 1], f[:, :, t:t + 1], *st1)
+        outs.append(h)
+    torch.testing.assert_close(torch.cat(outs, 2), H, rtol=1e-4, atol=1e-4)
+    for a, b in zip(st1, st):
+        torch.testing.assert_close(a, b, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("S", [128, 65, 1, 400])
+def test_pad_zeros_wrapper(S):
+    q, k, v, i, f = make_qkvif(1, 2, S, 32, 32, seed=S, dtype=torch.float64)
+    i, f = i.double(), f.double()
+    H = wrap_chunkwise__pad_zeros(O.mlstm_chunkwise__native_custbw, q=q, k=k, v=v, f=f, i=i, chunk_size=64)
+    H_ref, _ = O.recurrent_sequence(q, k, v, i, f)
+    assert H.shape == H_ref.shape
+    torch.testing.assert_close(H, H_ref, rtol=1e-8, atol=1e-8)
+    with pytest.raises(AssertionError):
+        wrap_chunkwise__pad_zeros(O.mlstm_chunkwise__native_custbw, q=q, k=k, v=v, f=f, i=i, return_last_states=True)

@@ -1,0 +1,90 @@
+"""Golden vectors: a hand-computed decode step and the committed chunkwise fixture.  On the CPU they pin the
+oracle (regression); on the GPU the HIP kernels are checked against the same files."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from helpers import allclose_frac, assert_state_close, rel_norm, rel_to_scale
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _kat():
+    return json.load(open(os.path.join(GOLD, "step_kat.json")))
+
+
+def _fixture():
+    z = np.load(os.path.join(GOLD, "chunkwise_small.npz"))
+    return {k: torch.from_numpy(z[k]) for k in z.files}
+
+
+def test_step_kat_oracle():
+    kat = _kat()
+    t = lambda x, *s: torch.full(s, x, dtype=torch.float64)
+    h, (c, n, m) = O.recurrent_step(t(kat["q"], 1, 1, 1), t(kat["k"], 1, 1, 1), t(kat["v"], 1, 1, 1), t(kat["i"], 1, 1, 1),
+                                    t(kat["f"], 1, 1, 1), t(kat["c"], 1, 1, 1, 1), t(kat["n"], 1, 1, 1), t(kat["m"], 1, 1, 1),
+                                    eps=kat["eps"])
+    assert abs(h.item() - kat["h"]) < 1e-12 and abs(c.item() - kat["c_new"]) < 1e-12
+    assert abs(n.item() - kat["n_new"]) < 1e-12 and abs(m.item() - kat["m_new"]) < 1e-15
+
+
+@pytest.mark.parametrize("tag,sig", [("exp", False), ("sig", True)])
+def test_chunkwise_fixture_oracle(tag, sig):
+    z = {k: v.double() for k, v in _fixture().items()}
+    fw = O.chunkwise_fw(z["q"], z["k"], z["v"], z["i"], z["f"], z["c0"], z["n0"], z["m0"], chunk_size=64, siging=sig)
+    bw = O.chunkwise_bw(z["q"], z["k"], z["v"], z["i"], z["f"], z["dH"], z["c0"], z["n0"], z["m0"], None, chunk_size=16, siging=sig)
+    torch.testing.assert_close(fw["H"], z[f"{tag}_H"], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(fw["C_last"], z[f"{tag}_C"], rtol=1e-5, atol=1e-5)
+    for name, t in zip(["dQ", "dK", "dV", "dI", "dF", "dC0"], bw):
+        torch.testing.assert_close(t, z[f"{tag}_{name}"], rtol=1e-4, atol=1e-4, msg=lambda s: f"{name}: {s}")
+
+
+@pytest.mark.gpu
+def test_step_kat_hip():
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip
+
+    kat = _kat()
+    # the kernel needs DHHV % 4 == 0: embed the scalar problem in column 0 / row 0 of zero-padded operands
+    dev = "cuda"
+    q = torch.zeros(1, 1, 4, device=dev); k = torch.zeros(1, 1, 4, device=dev); v = torch.zeros(1, 1, 4, device=dev)
+    q[..., 0], k[..., 0], v[..., 0] = kat["q"] * 2.0, kat["k"], kat["v"]   # q/sqrt(4) = kat q
+    c = torch.zeros(1, 1, 4, 4, device=dev); n = torch.zeros(1, 1, 4, device=dev)
+    c[..., 0, 0], n[..., 0] = kat["c"], kat["n"]
+    i = torch.full((1, 1, 1), kat["i"], device=dev); f = torch.full((1, 1, 1), kat["f"], device=dev)
+    m = torch.full((1, 1, 1), kat["m"], device=dev)
+    h, (c2, n2, m2) = mlstm_recurrent_step__hip(q, k, v, i, f, c, n, m, eps=kat["eps"])
+    assert abs(h[0, 0, 0].item() - kat["h"]) < 1e-5 * abs(kat["h"])
+    assert abs(c2[0, 0, 0, 0].item() - kat["c_new"]) < 1e-5 * kat["c_new"]
+    assert abs(n2[0, 0, 0].item() - kat["n_new"]) < 1e-6 and abs(m2.item() - kat["m_new"]) < 1e-6
+    assert h[0, 0, 1:].abs().max().item() == 0.0 and c2[0, 0, 1:, :].abs().max().item() == 0.0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag,sig", [("exp", False), ("sig", True)])
+def test_chunkwise_fixture_hip(tag, sig):
+    from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk
+
+    z = _fixture()
+    dev = "cuda"
+    q, k, v = (z[x].bfloat16().to(dev).requires_grad_(True) for x in "qkv")
+    i, f = z["i"].to(dev).requires_grad_(True), z["f"].to(dev).requires_grad_(True)
+    c0 = z["c0"].to(dev).requires_grad_(True)
+    fn = mlstm_siging_chunkwise__hip_xl_chunk if sig else mlstm_chunkwise__hip_xl_chunk
+    H, st = fn(q, k, v, i, f, c_initial=c0, n_initial=z["n0"].to(dev), m_initial=z["m0"].to(dev), return_last_states=True, chunk_size=128)
+    H.backward(z["dH"].bfloat16().to(dev))
+    # tolerances: outputs / gradients 2e-2 (bf16 operands), states 1e-3, gate gradients 5e-2 of their scale
+    assert allclose_frac(H, z[f"{tag}_H"], 2e-2, 2e-2) <= 1e-3 and rel_to_scale(H, z[f"{tag}_H"]) <= 1e-2
+    assert_state_close(st[0], z[f"{tag}_C"], 1e-3, "C_last")
+    assert_state_close(st[1], z[f"{tag}_n"], 1e-3, "n_last")
+    if not sig:
+        assert (st[2].cpu() - z["exp_m"]).abs().max() <= 1e-3
+    for name, t in (("dQ", q), ("dK", k), ("dV", v)):
+        assert allclose_frac(t.grad, z[f"{tag}_{name}"], 2e-2, 2e-2) <= 1e-3, name
+        assert rel_to_scale(t.grad, z[f"{tag}_{name}"]) <= 1e-2 and rel_norm(t.grad, z[f"{tag}_{name}"]) <= 5e-3, name
+    for name, t in (("dI", i), ("dF", f)):
+        assert rel_to_scale(t.grad, z[f"{tag}_{name}"]) <= 5e-2, name
+    assert rel_norm(c0.grad, z[f"{tag}_dC0"]) <= 5e-3

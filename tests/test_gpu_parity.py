@@ -1,0 +1,267 @@
+"""GPU parity tests: the HIP kernels (called through the C ABI via the operator wrappers) against the CPU
+oracle on the same seeded, bf16-rounded inputs.
+
+Stated tolerances (bf16 inputs, fp32 states):
+  * H, dQ, dK, dV: |x - ref| <= 2e-2 + 2e-2 |ref| element-wise.  The matrix kernels feed bf16-rounded operands
+    (gated scores, chunk states) to the matrix cores, so rows whose normaliser nearly cancels amplify a 2^-9
+    operand rounding beyond that bound on a few elements in 10^4; the tests therefore require the bound on
+    >= 99.9 % of the elements AND max|x - ref| <= 1e-2 max|ref| AND ||x - ref|| <= 5e-3 ||ref||.
+  * final C / n / m states: 1e-3 relative (max error over tensor scale, and norm-wise).
+  * dI, dF: 5e-2 of the tensor scale (sums over the head dimension / the whole sequence of differences of
+    bf16-rounded products; the reference's own tests allow atol 0.4 there).
+"""
+import pytest
+import torch
+
+import oracle as O
+from helpers import allclose_frac, assert_state_close, make_qkvif, rel_norm, rel_to_scale
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _ops():
+    from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_sequence__hip, mlstm_recurrent_step__hip
+
+    return mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk, mlstm_recurrent_step__hip, mlstm_recurrent_sequence__hip
+
+
+def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3):
+    bad = allclose_frac(x, ref, 2e-2, 2e-2)
+    e1, e2 = rel_to_scale(x, ref), rel_norm(x, ref)
+    assert bad <= frac and e1 <= scale_tol and e2 <= norm_tol, (
+        f"{name}: {bad:.2e} of elements outside 2e-2/2e-2, max err / scale {e1:.2e}, norm err {e2:.2e}")
+
+
+def d64(t):
+    return None if t is None else t.detach().double().cpu()
+
+
+# ------------------------------------------------------------------------------------------ decode step
+@pytest.mark.parametrize("B,NH,DQK,DHV", [(2, 2, 64, 128), (3, 4, 256, 512), (1, 1, 128, 192)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_step_parity(B, NH, DQK, DHV, dtype):
+    *_, step, _ = _ops()
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(B, NH, d, generator=g).to(dtype) for d in (DQK, DQK, DHV))
+    i, f = torch.randn(B, NH, 1, generator=g), 3 + torch.randn(B, NH, 1, generator=g)
+    c, n, m = torch.randn(B, NH, DQK, DHV, generator=g), torch.randn(B, NH, DQK, generator=g), torch.randn(B, NH, 1, generator=g)
+    h_r, (c_r, n_r, m_r) = O.recurrent_step(*(d64(t) for t in (q, k, v, i, f, c, n, m)))
+    h, (c2, n2, m2) = step(*(t.to(DEV) for t in (q, k, v, i, f, c, n, m)))
+    assert h.dtype == dtype and c2.dtype == torch.float32
+    assert rel_to_scale(h, h_r) <= (5e-3 if dtype == torch.bfloat16 else 1e-5)
+    assert_state_close(c2, c_r, 1e-5, "C")
+    assert_state_close(n2, n_r, 1e-5, "n")
+    assert (d64(m2) - m_r).abs().max() <= 1e-5
+    # in-place update of C gives the same result
+    c_dev = c.to(DEV).clone()
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw
+    n_new, m_new = torch.empty_like(n2), torch.empty_like(m2)
+    h3, (c3, _, _) = mlstm_recurrent_step__hip_fw(c_dev, n.to(DEV), m.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), i.to(DEV), f.to(DEV),
+                                                  matC_new=c_dev, vecN_new=n_new, scaM_new=m_new)
+    assert c3.data_ptr() == c_dev.data_ptr() and torch.equal(c3, c2) and torch.equal(h3, h)
+
+
+def test_decode_after_prefill():
+    """Prefill S=2048 with the chunkwise kernel, then 128 consecutive decode steps (state updated in place);
+    the oracle does the same in fp64 for the first two batch rows."""
+    exp_op, _, step, _ = _ops()
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw
+    B, NH, S, DQK, DHV, T = 16, 8, 2048, 256, 512, 128
+    Bo = 2
+    q, k, v, i, f = make_qkvif(B, NH, S, DQK, DHV, seed=0)
+    _, (c, n, m) = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
+    ref = O.chunkwise_fw(*(d64(t[:Bo]) for t in (q, k, v, i, f)), chunk_size=128)
+    c_r, n_r, m_r = ref["C_last"], ref["n_last"], ref["m_last"]
+    assert_state_close(c[:Bo], c_r, 1e-3, "prefill C")
+    g = torch.Generator().manual_seed(1)
+    n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
+    worst_h = 0.0
+    for t in range(T):
+        qt, kt, vt = (torch.randn(B, NH, d, generator=g).bfloat16() for d in (DQK, DQK, DHV))
+        it, ft = torch.randn(B, NH, 1, generator=g), 3 + torch.randn(B, NH, 1, generator=g)
+        h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(c, n, m, qt.to(DEV), kt.to(DEV), vt.to(DEV), it.to(DEV), ft.to(DEV),
+                                                           matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
+        n_alt, m_alt, n, m = n, m, n_new, m_new
+        h_r, (c_r, n_r, m_r) = O.recurrent_step(*(d64(x[:Bo]) for x in (qt, kt, vt, it, ft)), c_r, n_r, m_r)
+        worst_h = max(worst_h, allclose_frac(h[:Bo], h_r, 2e-2, 2e-2))
+    assert worst_h == 0.0, f"h outside 2e-2/2e-2 on a fraction {worst_h} of elements"
+    assert_state_close(c[:Bo], c_r, 1e-3, "C after 128 steps")
+    assert_state_close(n[:Bo], n_r, 1e-3, "n after 128 steps")
+    assert (d64(m[:Bo]) - m_r).abs().max() <= 1e-3
+
+
+# ------------------------------------------------------------------------------------------ chunkwise forward
+@pytest.mark.parametrize("cfg", [
+    dict(B=1, NH=4, S=256, DQK=64, DHV=64, L=64, seed=0, dtype=torch.float32),    # BASELINE config 1 shape
+    dict(B=2, NH=4, S=512, DQK=128, DHV=256, L=256, seed=1, dtype=torch.bfloat16),  # BASELINE config 2
+    dict(B=1, NH=2, S=144, DQK=64, DHV=128, L=16, seed=2, dtype=torch.bfloat16),   # ragged tail (128 + 16)
+    dict(B=1, NH=2, S=32, DQK=64, DHV=64, L=32, seed=3, dtype=torch.bfloat16),     # shorter than one chunk
+    dict(B=1, NH=1, S=256, DQK=256, DHV=1024, L=128, seed=4, dtype=torch.bfloat16),  # several value-column tiles
+])
+def test_chunkwise_forward_exp(cfg):
+    exp_op, *_ = _ops()
+    q, k, v, i, f = make_qkvif(cfg["B"], cfg["NH"], cfg["S"], cfg["DQK"], cfg["DHV"], cfg["seed"])
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=min(cfg["L"], 64))
+    args = [t.to(DEV) for t in (q.to(cfg["dtype"]), k.to(cfg["dtype"]), v.to(cfg["dtype"]), i, f)]
+    H, (C, n, m) = exp_op(*args, return_last_states=True, chunk_size=cfg["L"])
+    assert H.dtype == cfg["dtype"] and H.shape == v.shape and C.dtype == torch.float32
+    assert m.shape == (cfg["B"], cfg["NH"], 1)
+    check_matrix(H, ref["H"], "H")
+    assert_state_close(C, ref["C_last"], 1e-3, "C_last")
+    assert_state_close(n, ref["n_last"], 1e-3, "n_last")
+    assert (d64(m) - ref["m_last"]).abs().max() <= 1e-3
+    H2 = exp_op(*args, return_last_states=False, chunk_size=cfg["L"])
+    assert torch.equal(H2, H)
+
+
+@pytest.mark.parametrize("f_offset", [0.0, -3.0, 6.0])
+def test_chunkwise_forward_gate_regimes(f_offset):
+    exp_op, *_ = _ops()
+    q, k, v, i, f = make_qkvif(1, 2, 384, 64, 128, seed=7, f_offset=f_offset)
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=64)
+    H, (C, n, m) = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
+    check_matrix(H, ref["H"], "H", frac=2e-3)
+    assert_state_close(C, ref["C_last"], 1e-3, "C_last")
+    assert (d64(m) - ref["m_last"]).abs().max() <= 1e-3
+
+
+def test_unsupported_head_dim_fails_loudly():
+    exp_op, *_ = _ops()
+    q, k, v, i, f = make_qkvif(1, 1, 128, 512, 128)
+    with pytest.raises(RuntimeError, match="DHQK too large"):
+        exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128)
+    q, k, v, i, f = make_qkvif(1, 1, 128, 96, 128)
+    with pytest.raises(ValueError, match="multiples of 64"):
+        exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128)
+
+
+# ------------------------------------------------------------------------------------------ forward + backward
+def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl=False, seed=0, pairs=None, L=128):
+    exp_op, sig_op, *_ = _ops()
+    gpu_gen = torch.Generator(device=DEV).manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gpu_gen)
+    q, k, v, dH = rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DHV).bfloat16(), rn(B, NH, S, DHV).bfloat16()
+    i, f = rn(B, NH, S), 3 + rn(B, NH, S)
+    c0 = n0 = m0 = dCl = None
+    if init:
+        c0, n0, m0 = 0.1 * rn(B, NH, DQK, DHV), 0.1 * rn(B, NH, DQK), torch.zeros(B, NH, 1, device=DEV)
+    if dcl:
+        dCl = 0.1 * rn(B, NH, DQK, DHV)
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, i, f)]
+    c0l = None if c0 is None else c0.clone().requires_grad_(True)
+    kw = dict(c_initial=c0l, n_initial=n0, m_initial=m0, return_last_states=True, chunk_size=L)
+    if siging:
+        H, st = sig_op(*leaves, normalize=normalize, **kw)
+    else:
+        H, st = exp_op(*leaves, **kw)
+    loss = (H.float() * dH.float()).sum()
+    if dCl is not None:
+        loss = loss + (st[0] * dCl).sum()
+    loss.backward()
+    # oracle on a subset of (batch, head) pairs: every pair is independent
+    pairs = pairs or [(b, h) for b in range(B) for h in range(NH)]
+    Lo = next(c for c in (128, 64, 32, 16) if S % c == 0)   # the oracle's chunk length (results do not depend on it)
+    for (b, h) in pairs:
+        sl = lambda t: None if t is None else d64(t[b:b + 1, h:h + 1])
+        fw = O.chunkwise_fw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(c0), sl(n0), sl(m0), chunk_size=Lo, siging=siging, normalize=normalize)
+        bw = O.chunkwise_bw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(dH), sl(c0), sl(n0), sl(m0), sl(dCl), chunk_size=Lo, siging=siging, normalize=normalize)
+        tag = f"(b={b},h={h})"
+        check_matrix(H[b:b + 1, h:h + 1], fw["H"], "H" + tag)
+        assert_state_close(st[0][b:b + 1, h:h + 1], fw["C_last"], 1e-3, "C_last" + tag)
+        assert_state_close(st[1][b:b + 1, h:h + 1], fw["n_last"], 1e-3, "n_last" + tag)
+        if not siging:
+            assert (d64(st[2][b:b + 1, h:h + 1]) - fw["m_last"]).abs().max() <= 1e-3
+        for name, leaf, r in zip(["dQ", "dK", "dV"], leaves[:3], bw[:3]):
+            check_matrix(leaf.grad[b:b + 1, h:h + 1], r, name + tag)
+        for name, leaf, r in zip(["dI", "dF"], leaves[3:], bw[3:5]):
+            e = rel_to_scale(leaf.grad[b:b + 1, h:h + 1], r)
+            assert e <= 5e-2, f"{name}{tag}: max err / scale {e:.2e}"
+        if c0l is not None:
+            assert rel_norm(c0l.grad[b:b + 1, h:h + 1], bw[5]) <= 5e-3, "dC0" + tag
+
+
+@pytest.mark.parametrize("kw", [
+    dict(B=1, NH=2, S=256, DQK=64, DHV=128),
+    dict(B=2, NH=2, S=512, DQK=128, DHV=256, seed=1),
+    dict(B=1, NH=2, S=384, DQK=256, DHV=512, init=True, dcl=True),
+    dict(B=1, NH=2, S=256, DQK=64, DHV=128, siging=True, init=True),
+    dict(B=1, NH=2, S=256, DQK=64, DHV=64, siging=True, normalize=False),
+    dict(B=1, NH=2, S=144, DQK=64, DHV=64, L=16),                  # ragged tail
+])
+def test_chunkwise_fwbw_small(kw):
+    _fwbw_case(**kw)
+
+
+@pytest.mark.parametrize("B,S", [(64, 1024), (16, 4096), (4, 16384)])
+def test_chunkwise_fwbw_xlstm7b_shape_exp(B, S):
+    """BASELINE config 3: NH=8, DHQK=256, DHHV=512, B*S = 65536, upstream dH ~ N(0,1).  The whole tensor runs on
+    the GPU; two (batch, head) pairs are checked against the fp64 oracle over the full sequence."""
+    _fwbw_case(B, 8, S, 256, 512, seed=0, pairs=[(0, 0), (B - 1, 5)])
+
+
+def test_chunkwise_fwbw_xlstm7b_shape_sig():
+    """BASELINE config 4: mLSTMsig, B=4, S=16384, non-zero initial C ~ N(0,0.1), n ~ N(0,0.1), m = 0."""
+    _fwbw_case(4, 8, 16384, 256, 512, siging=True, init=True, seed=0, pairs=[(1, 3), (3, 7)])
+
+
+# ------------------------------------------------------------------------------------------ size-independent properties
+def test_state_passing_and_exact_value_scaling_at_full_size():
+    exp_op, *_ = _ops()
+    B, NH, S, DQK, DHV = 4, 8, 8192, 256, 512
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    q, k, v = rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DHV).bfloat16()
+    i, f = rn(B, NH, S), 3 + rn(B, NH, S)
+    H, (C, n, m) = exp_op(q, k, v, i, f, return_last_states=True, chunk_size=128)
+    # (a) two calls threading (C, n, m) reproduce one call
+    cut = 3072
+    H1, st1 = exp_op(q[:, :, :cut].contiguous(), k[:, :, :cut].contiguous(), v[:, :, :cut].contiguous(),
+                     i[:, :, :cut].contiguous(), f[:, :, :cut].contiguous(), return_last_states=True, chunk_size=128)
+    H2, (C2, n2, m2) = exp_op(q[:, :, cut:].contiguous(), k[:, :, cut:].contiguous(), v[:, :, cut:].contiguous(),
+                              i[:, :, cut:].contiguous(), f[:, :, cut:].contiguous(), *st1, return_last_states=True, chunk_size=128)
+    assert torch.equal(H1, H[:, :, :cut])
+    Hc = torch.cat([H1, H2], 2)
+    assert allclose_frac(Hc, H, 2e-2, 2e-2) <= 1e-3 and rel_norm(Hc, H) <= 5e-3
+    assert_state_close(C2, C, 1e-3, "C_last")
+    assert_state_close(n2, n, 1e-3, "n_last")
+    assert (m2 - m).abs().max().item() <= 1e-4
+    # (b) doubling v doubles H and C exactly (powers of two commute with every rounding), n and m unchanged
+    Hd, (Cd, nd, md) = exp_op(q, k, (v.float() * 2).bfloat16(), i, f, return_last_states=True, chunk_size=128)
+    assert torch.equal(Hd.float(), H.float() * 2) and torch.equal(Cd, C * 2) and torch.equal(nd, n) and torch.equal(md, m)
+    assert not torch.isnan(H.float()).any()
+
+
+# ------------------------------------------------------------------------------------------ backend module on the GPU
+def test_backend_module_hip_train_and_inference():
+    from mlstm_kernels_amd.torch.backend_module import mLSTMBackend, mLSTMBackendConfig
+
+    q, k, v, i, f = make_qkvif(2, 2, 293, 64, 128, seed=11)   # 293 = 2*128 + 32 + 5: chunks, a halved chunk, token loop
+    ref_H, (c_r, n_r, m_r) = O.recurrent_sequence(*(d64(t) for t in (q, k, v, i, f)))
+    backend = mLSTMBackend(mLSTMBackendConfig(chunk_size=128, mode="inference")).to(DEV)
+    H, (C, n, m) = backend(*(t.to(DEV) for t in (q, k, v, i, f)))
+    assert H.dtype == q.dtype and H.shape == v.shape
+    check_matrix(H, ref_H, "H (inference, arbitrary length)", frac=2e-3)
+    assert_state_close(C, c_r, 1e-3, "C")
+    # one generation step from those states goes through the HIP step kernel
+    g = torch.Generator().manual_seed(2)
+    q1, k1, v1 = (torch.randn(2, 2, 1, d, generator=g).bfloat16() for d in (64, 64, 128))
+    i1, f1 = torch.randn(2, 2, 1, generator=g), 3 + torch.randn(2, 2, 1, generator=g)
+    h1, (C1, n1, m1) = backend(*(t.to(DEV) for t in (q1, k1, v1, i1, f1)), C, n, m)
+    h1_r, (c1_r, _, _) = O.recurrent_step(d64(q1[:, :, 0]), d64(k1[:, :, 0]), d64(v1[:, :, 0]), d64(i1), d64(f1), c_r, n_r, m_r)
+    assert h1.shape == (2, 2, 1, 128) and allclose_frac(h1[:, :, 0], h1_r, 2e-2, 2e-2) == 0.0
+    assert_state_close(C1, c1_r, 1e-3, "C after step")
+    # train mode, padded train mode, sigmoid gate through the module
+    train = mLSTMBackend(mLSTMBackendConfig(chunk_size=128, mode="train"))
+    qq, kk, vv, ii, ff = (t[:, :, :256].contiguous().to(DEV) for t in (q, k, v, i, f))
+    Ht, (Ct, nt, mt) = train(qq, kk, vv, ii, ff)
+    check_matrix(Ht, ref_H[:, :, :256], "H (train)")
+    padded = mLSTMBackend(mLSTMBackendConfig(chunk_size=128, mode="train_with_padding", return_last_states=False))
+    Hp = padded(*(t[:, :, :200].contiguous().to(DEV) for t in (q, k, v, i, f)))
+    assert Hp.shape == (2, 2, 200, 128)
+    check_matrix(Hp, ref_H[:, :, :200], "H (padded)")
+    sig = mLSTMBackend(mLSTMBackendConfig(chunkwise_kernel="chunkwise--hip_xl_chunk_siging", chunk_size=128, normalize_siging=False))
+    Hs, (Cs, ns) = sig(qq, kk, vv, ii, ff)
+    Hs_r, _ = O.parallel_siging_fw(*(d64(t[:, :, :256]) for t in (q, k, v, i, f)), normalize=False)
+    check_matrix(Hs, Hs_r, "H (sig, not normalised)")
