@@ -4,7 +4,8 @@
  *
  * Conventions
  *   - Every pointer is a DEVICE pointer owned by the caller; the library never allocates or frees device
- *     memory and keeps no state between calls except a thread-local error string.
+ *     memory and keeps no state between calls except a thread-local error string (and, while the optional
+ *     per-kernel timing is enabled, host-side event records).
  *   - Tensors are dense row-major: q,k (B,NH,S,DHQK); v,H,dH (B,NH,S,DHHV); i,f (B,NH,S);
  *     C (B,NH,DHQK,DHHV) fp32; n (B,NH,DHQK) fp32; m (B,NH) fp32.
  *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it.
@@ -33,6 +34,16 @@ extern "C" {
 /* ABI version of the loaded library (bumped on any signature change). */
 int mlstm_hip_abi_version(void);
 
+/*
+ * Per-kernel timing for benchmarks (no counterpart in the reference, which times whole operator calls with
+ * torch events: mlstm_kernels/utils/benchmark/runtime.py:30-170).  While enabled, every kernel launch of this
+ * library is bracketed by HIP events on its launch stream.  mlstm_hip_profile_read(0, ...) waits for the
+ * recorded events, aggregates them by kernel name and returns the number of distinct kernels; entry `index`
+ * (name, summed milliseconds, number of launches) is copied out.  Host-side bookkeeping only.
+ */
+int mlstm_hip_profile_enable(int on);
+int mlstm_hip_profile_read(int index, char* name, size_t name_cap, float* total_ms, int* launches);
+
 /* Message of the last failure on the calling thread ("" if none). */
 const char* mlstm_hip_last_error(void);
 
@@ -41,7 +52,8 @@ const char* mlstm_hip_last_error(void);
  * Replaces: mlstm_kernels/torch/recurrent/triton_step.py:15-127 (mlstm_recurrent_step__triton_fw) and the
  * Triton kernel mlstm_kernels/triton/recurrent/fw_step_fused.py:19-195.
  *   q,k (B,NH,DHQK), v (B,NH,DHHV) in dtype_qkv; i,f (B,NH) in dtype_gates; h (B,NH,DHHV) in dtype_qkv.
- *   c_out/n_out/m_out may alias c_in/n_in/m_in (in-place update) or be distinct buffers.
+ *   c_out may alias c_in (in-place update of the state matrix); n_out/m_out must be distinct from n_in/m_in
+ *   (every workgroup of a head reads the old n and m while one of them writes the new values).
  */
 int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f,
                    const float* c_in, const float* n_in, const float* m_in,

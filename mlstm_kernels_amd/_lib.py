@@ -18,6 +18,8 @@ _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_
 _SIGNATURES = {
     "mlstm_hip_abi_version": (_i, []),
     "mlstm_hip_last_error": (ctypes.c_char_p, []),
+    "mlstm_hip_profile_enable": (_i, [_i]),
+    "mlstm_hip_profile_read": (_i, [_i, ctypes.c_char_p, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)]),
     "mlstm_hip_step": (_i, [_vp] * 12 + [_i, _i, _i, _i, _f, _i, _i, _vp]),
     "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 6),
     "mlstm_hip_chunkwise_fw": (_i, [_vp] * 15 + [_sz, _i] + [_i] * 5 + [_f] + [_i] * 4 + [_vp]),
@@ -57,6 +59,24 @@ def get_lib() -> ctypes.CDLL:
                 )
             _lib = lib
     return _lib
+
+
+def profile_enable(on: bool) -> None:
+    get_lib().mlstm_hip_profile_enable(int(on))
+
+
+def profile_read() -> dict[str, tuple[float, int]]:
+    """{kernel name: (summed milliseconds, launches)} of everything recorded since the last read."""
+    lib = get_lib()
+    out: dict[str, tuple[float, int]] = {}
+    buf = ctypes.create_string_buffer(64)
+    ms, cnt = ctypes.c_float(0.0), ctypes.c_int(0)
+    n = lib.mlstm_hip_profile_read(0, buf, 64, ctypes.byref(ms), ctypes.byref(cnt))  # index 0 aggregates
+    for idx in range(n):
+        if idx > 0:
+            lib.mlstm_hip_profile_read(idx, buf, 64, ctypes.byref(ms), ctypes.byref(cnt))
+        out[buf.value.decode()] = (ms.value, cnt.value)
+    return out
 
 
 def check(rc: int, what: str) -> None:

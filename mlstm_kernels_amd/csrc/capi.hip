@@ -4,11 +4,44 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <string>
+#include <vector>
+
 #include "../../include/mlstm_hip.h"
 #include "kernels.h"
 
 namespace {
 thread_local char g_err[512] = "";
+
+// Optional per-kernel timing: when enabled, every kernel launch issued by this library is bracketed by a
+// pair of HIP events recorded on the launch stream.  Host-side bookkeeping only; no device memory.
+struct TimedLaunch {
+  const char* name;
+  hipEvent_t start, stop;
+};
+std::mutex g_prof_mutex;
+bool g_prof_on = false;
+std::vector<TimedLaunch> g_prof_launches;
+
+struct ProfileScope {
+  const char* name;
+  hipStream_t stream;
+  hipEvent_t start = nullptr, stop = nullptr;
+  bool active = false;
+  ProfileScope(const char* n, hipStream_t s) : name(n), stream(s) {
+    if (!g_prof_on) return;
+    if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return;
+    active = true;
+    (void)hipEventRecord(start, stream);
+  }
+  ~ProfileScope() {
+    if (!active) return;
+    (void)hipEventRecord(stop, stream);
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    g_prof_launches.push_back({name, start, stop});
+  }
+};
 int fail(const char* msg) {
   snprintf(g_err, sizeof(g_err), "%s", msg);
   return 1;
@@ -32,6 +65,43 @@ const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {
 extern "C" {
 
 int mlstm_hip_abi_version(void) { return 1; }
+
+int mlstm_hip_profile_enable(int on) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof_on = on != 0;
+  return 0;
+}
+
+int mlstm_hip_profile_read(int index, char* name, size_t name_cap, float* total_ms, int* launches) {
+  // Aggregates the recorded launches by kernel name (first call of a read-out pass: index 0), waits for their
+  // events, and returns the number of distinct kernels; entry `index` is copied out when it exists.
+  static std::vector<std::string> names;
+  static std::vector<float> totals;
+  static std::vector<int> counts;
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  if (index == 0) {
+    names.clear(); totals.clear(); counts.clear();
+    for (TimedLaunch& t : g_prof_launches) {
+      float ms = 0.f;
+      if (hipEventSynchronize(t.stop) == hipSuccess) (void)hipEventElapsedTime(&ms, t.start, t.stop);
+      (void)hipEventDestroy(t.start);
+      (void)hipEventDestroy(t.stop);
+      size_t k = 0;
+      for (; k < names.size(); ++k)
+        if (names[k] == t.name) break;
+      if (k == names.size()) { names.push_back(t.name); totals.push_back(0.f); counts.push_back(0); }
+      totals[k] += ms;
+      counts[k] += 1;
+    }
+    g_prof_launches.clear();
+  }
+  if (index >= 0 && (size_t)index < names.size()) {
+    if (name && name_cap) snprintf(name, name_cap, "%s", names[index].c_str());
+    if (total_ms) *total_ms = totals[index];
+    if (launches) *launches = counts[index];
+  }
+  return (int)names.size();
+}
 const char* mlstm_hip_last_error(void) { return g_err; }
 
 int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c_in,
@@ -43,9 +113,12 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
     return fail("mlstm_hip_step: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
   if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16))
     return fail("mlstm_hip_step: unsupported dtype code");
-  const char* e = mlstm::launch_step(q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps,
-                                     dtype_qkv, dtype_gates, (hipStream_t)stream);
-  if (e) return fail(e);
+  {
+    ProfileScope ps("step", (hipStream_t)stream);
+    const char* e = mlstm::launch_step(q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps,
+                                       dtype_qkv, dtype_gates, (hipStream_t)stream);
+    if (e) return fail(e);
+  }
   return check_launch("mlstm_hip_step");
 }
 
@@ -75,7 +148,10 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   hipStream_t st = (hipStream_t)stream;
   const int NC = (S + 127) / 128, BH = B * NH;
   const int sig = gate == MLSTM_GATE_SIG;
-  if (const char* e = mlstm::launch_gates(i, f, m0, ws.g, m_last, B, NH, S, dtype_gates, sig, st)) return fail(e);
+  {
+    ProfileScope ps("gates", st);
+    if (const char* e = mlstm::launch_gates(i, f, m0, ws.g, m_last, B, NH, S, dtype_gates, sig, st)) return fail(e);
+  }
   if (check_launch("gates")) return 1;
 
   mlstm::ScanArgs sa;
@@ -103,7 +179,10 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   sa.qk_scale = 1.0f / sqrtf((float)DHQK);
   sa.eps = eps;
   sa.backward = 0;
-  if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/true, st)) return fail(e);
+  {
+    ProfileScope ps("scan_fw", st);
+    if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/true, st)) return fail(e);
+  }
   if (check_launch("scan_fw")) return 1;
 
   mlstm::ParHvArgs pa;
@@ -119,7 +198,10 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   pa.qk_scale = sa.qk_scale; pa.eps = eps;
   pa.sig_gate = sig;
   pa.use_nrow = !(sig && !normalize);
-  if (const char* e = mlstm::launch_par_hv(pa, BH, /*is_dv=*/false, st)) return fail(e);
+  {
+    ProfileScope ps("par_h", st);
+    if (const char* e = mlstm::launch_par_hv(pa, BH, /*is_dv=*/false, st)) return fail(e);
+  }
   return check_launch("par_hv forward");
 }
 
@@ -162,7 +244,10 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   sa.S = S; sa.NC = NC; sa.DHQK = DHQK; sa.DHHV = DHHV;
   sa.qk_scale = qk_scale; sa.eps = eps;
   sa.backward = 1;
-  if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/false, st)) return fail(e);
+  {
+    ProfileScope ps("scan_bw", st);
+    if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/false, st)) return fail(e);
+  }
   if (check_launch("scan_bw")) return 1;
 
   mlstm::ParHvArgs pv;
@@ -175,7 +260,10 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   pv.S = S; pv.NC = NC; pv.DHQK = DHQK; pv.DHHV = DHHV;
   pv.qk_scale = qk_scale; pv.eps = eps;
   pv.sig_gate = sig; pv.use_nrow = use_nrow;
-  if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
+  {
+    ProfileScope ps("par_dv", st);
+    if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
+  }
   if (check_launch("par_hv dV")) return 1;
 
   const int MT = DHQK % 256 == 0 ? 256 : (DHQK % 128 == 0 ? 128 : 64);
@@ -193,17 +281,26 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   pq.qk_scale = qk_scale; pq.eps = eps;
   pq.use_nrow = use_nrow;
   pq.states = ws.cstates; pq.Out = (uint16_t*)dQ; pq.rowdot = bws.qdq;
-  if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/true, st)) return fail(e);
+  {
+    ProfileScope ps("par_dq", st);
+    if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/true, st)) return fail(e);
+  }
   if (check_launch("par_qk dQ")) return 1;
   pq.states = bws.dcstates; pq.Out = (uint16_t*)dK; pq.rowdot = bws.kdk;
-  if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/false, st)) return fail(e);
+  {
+    ProfileScope ps("par_dk", st);
+    if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/false, st)) return fail(e);
+  }
   if (check_launch("par_qk dK")) return 1;
 
   mlstm::GateGradArgs ga;
   memset(&ga, 0, sizeof(ga));
   ga.i = i; ga.f = f; ga.qdq = bws.qdq; ga.kdk = bws.kdk; ga.dI = dI; ga.dF = dF;
   ga.S = S; ga.NC = NC; ga.dtype_gates = dtype_gates; ga.sig_gate = sig;
-  if (const char* e = mlstm::launch_gate_grads(ga, BH, st)) return fail(e);
+  {
+    ProfileScope ps("gate_grads", st);
+    if (const char* e = mlstm::launch_gate_grads(ga, BH, st)) return fail(e);
+  }
   return check_launch("gate_grads");
 }
 
