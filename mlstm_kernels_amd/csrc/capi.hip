@@ -2,6 +2,7 @@
 // kernel sequencing.  No device memory is allocated here and no state is kept between calls.
 #include <hip/hip_runtime.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>

@@ -32,8 +32,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   u += 0x7fffu + ((u >> 16) & 1u);
   return (uint16_t)(u >> 16);
 }
+// two fp32 -> packed bf16x2 (round to nearest even) with the gfx950 hardware conversion v_cvt_pk_bf16_f32
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  const f32x2_hw v = {lo, hi};
+  const bf16x2_hw b = __builtin_convertvector(v, bf16x2_hw);
+  uint32_t u;
+  __builtin_memcpy(&u, &b, 4);
+  return u;
 }
 
 // D(32x32) += A(32x16) * B(16x32), bf16 operands, fp32 accumulate.
@@ -72,6 +79,25 @@ __device__ __forceinline__ float log_sigmoid(float x) {
 
 __device__ __forceinline__ float load_scalar(const void* p, size_t idx, int dtype) {
   return dtype == 0 ? ((const float*)p)[idx] : bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+}
+
+// XCD-aware workgroup renumbering.  The hardware deals consecutive linear workgroup ids round-robin to the 8
+// XCDs (each with its own L2).  Mapping linear id -> (id % 8) * (total / 8) + id / 8 gives every XCD a
+// contiguous range of virtual ids, so neighbouring tiles (which share operands) share an L2.
+struct BlockId {
+  int x, y, z;
+};
+__device__ __forceinline__ BlockId xcd_block_id() {
+  BlockId b = {(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z};
+  const int gx = gridDim.x, gy = gridDim.y, total = gx * gy * (int)gridDim.z;
+  if (total % 8 == 0) {
+    const int lin = b.x + gx * (b.y + gy * b.z);
+    const int virt = (lin % 8) * (total / 8) + lin / 8;
+    b.x = virt % gx;
+    b.y = (virt / gx) % gy;
+    b.z = virt / (gx * gy);
+  }
+  return b;
 }
 
 // LDS write of one 16-byte global vector (8 consecutive head-dim entries) in the fragment order used for

@@ -48,8 +48,9 @@ __global__ __launch_bounds__(256) void par_hv_kernel(ParHvArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int mi = wave >> 1, ni = wave & 1;
   const int r = lane & 31, h = lane >> 5;
-  const int bh = blockIdx.z, c = blockIdx.y;
-  const int w_tile = blockIdx.x * WT;
+  const BlockId blk = xcd_block_id();  // the column tiles of one chunk share Q, K: keep them on one XCD
+  const int bh = blk.z, c = blk.y;
+  const int w_tile = blk.x * WT;
   const size_t Sp = (size_t)NC * kChunk;
   const size_t gofs = bh * Sp + (size_t)c * kChunk;
   const int t_base = c * kChunk;
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(256) void par_hv_kernel(ParHvArgs a) {
         iv = 1.f / (nmax + a.eps);
       }
       inv[t] = iv;
-      if (blockIdx.x == 0) {
+      if (blk.x == 0) {
         a.nrow_out[gofs + t] = nmax;
         if (t_base + t < S) {
           if (a.n_out != nullptr) a.n_out[(size_t)bh * S + t_base + t] = nmax;

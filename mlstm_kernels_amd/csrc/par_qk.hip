@@ -46,8 +46,9 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int mi = wave >> 1, ni = wave & 1;
   const int r = lane & 31, h = lane >> 5;
-  const int bh = blockIdx.z, c = blockIdx.y;
-  const int d_tile = blockIdx.x * MT;
+  const BlockId blk = xcd_block_id();
+  const int bh = blk.z, c = blk.y;
+  const int d_tile = blk.x * MT;
   const size_t Sp = (size_t)NC * kChunk;
   const size_t gofs = bh * Sp + (size_t)c * kChunk;
   const int t_base = c * kChunk;

@@ -15,11 +15,14 @@
 // forward the scaled rows are split into a bf16 head and a bf16 remainder (two MFMAs) so that the final
 // state keeps ~16 mantissa bits: a single bf16 rounding of abar*V leaves a relative error of about 1.5e-3
 // in C, above the 1e-3 the state is specified to.
+//
+// Workgroups are renumbered so that all tiles of one (batch, head) run on the same XCD (the hardware deals
+// consecutive workgroup ids round-robin to the 8 XCDs): the K/V rows every tile of a head re-reads then hit
+// that XCD's L2 instead of going to HBM once per tile.
 #include "common.h"
 #include "kernels.h"
 
 namespace mlstm {
-
 
 template <int RT, int WT, bool HILO>
 __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanArgs a) {
@@ -29,17 +32,30 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   constexpr int YS = WT + 16;
   constexpr int XV = 128 * RT / 8 / NT;  // 16-byte vectors per thread per chunk
   constexpr int YV = 128 * WT / 8 / NT;
+  constexpr int XROWS = NT / (RT / 8);   // rows covered by one sweep of the workgroup over X
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint16_t* Xs = (uint16_t*)smem_raw;
   uint16_t* Yh = Xs + 128 * XS;
   uint16_t* Yl = Yh + 128 * YS;
-  float* sc = (float*)(Yl + (HILO ? 128 * YS : 0));  // [128] row scale of the current chunk
+  float* npart = (float*)(Yl + (HILO ? 128 * YS : 0));  // [XROWS][RT] partial sums of the n update
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wr = wave / WC, wc = wave % WC;
   const int r = lane & 31, h = lane >> 5;
-  const int bh = blockIdx.z;
-  const int d_tile = blockIdx.x * RT, w_tile = blockIdx.y * WT;
+  // ---- XCD-aware renumbering: linear id -> (xcd, slot) -> contiguous range of ids per XCD
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  {
+    const int total = gridDim.x * gridDim.y * gridDim.z;
+    if (total % 8 == 0) {
+      const int lin = bx + gridDim.x * (by + gridDim.y * bz);
+      const int virt = (lin % 8) * (total / 8) + lin / 8;
+      bx = virt % gridDim.x;
+      by = (virt / gridDim.x) % gridDim.y;
+      bz = virt / (gridDim.x * gridDim.y);
+    }
+  }
+  const int bh = bz;
+  const int d_tile = bx * RT, w_tile = by * WT;
   const int d_wave = d_tile + wr * 64, w_wave = w_tile + wc * 64;
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   const size_t Sp = (size_t)NC * kChunk;
@@ -60,15 +76,24 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
         acc[db][wb][i] = v0;
       }
     }
-  const bool do_n = (a.nstates != nullptr) && blockIdx.y == 0 && tid < RT;
+  const bool do_n = (a.nstates != nullptr) && by == 0;
   float nval = 0.f;
-  if (do_n && a.n_init != nullptr) nval = a.n_init[(size_t)bh * DHQK + d_tile + tid];
+  if (do_n && tid < RT && a.n_init != nullptr) nval = a.n_init[(size_t)bh * DHQK + d_tile + tid];
 
   const uint16_t* Xg = a.X + (size_t)bh * S * DHQK + d_tile;
   const uint16_t* Yg = a.Y + (size_t)bh * S * DHHV + w_tile;
 
   uint4 xr[XV], yr[YV];
-  float ysc[YV];
+  float xsc[XV], ysc[YV];
+  auto row_scale = [&](int t) -> float {
+    if (t >= S) return 0.f;
+    float s = a.scale_a[bh * Sp + t];
+    if (a.backward) {
+      s *= a.qk_scale;
+      if (a.nrow != nullptr) s /= (a.nrow[bh * Sp + t] + a.eps);
+    }
+    return s;
+  };
   auto prefetch = [&](int c) {
 #pragma unroll
     for (int v = 0; v < XV; ++v) {
@@ -76,6 +101,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       const int j = idx / (RT / 8), cv = idx % (RT / 8);
       const int t = c * kChunk + j;
       xr[v] = t < S ? *(const uint4*)(Xg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
+      if (do_n) xsc[v] = row_scale(t);
     }
 #pragma unroll
     for (int v = 0; v < YV; ++v) {
@@ -83,12 +109,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
       const int t = c * kChunk + j;
       yr[v] = t < S ? *(const uint4*)(Yg + (size_t)t * DHHV + cv * 8) : make_uint4(0, 0, 0, 0);
-      float s = a.scale_a[bh * Sp + t];
-      if (a.backward) {
-        s *= a.qk_scale;
-        if (a.nrow != nullptr) s /= (a.nrow[bh * Sp + t] + a.eps);
-      }
-      ysc[v] = t < S ? s : 0.f;
+      ysc[v] = row_scale(t);
     }
   };
 
@@ -96,12 +117,27 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   prefetch(c_first);
   for (int it = 0; it < NC; ++it) {
     const int c = c_first + it * c_step;
-    // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split)
+    // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split); partial sums of sum_j abar_j k_j
+    float np[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int v = 0; v < XV; ++v) {
       const int idx = tid + v * NT;
       const int j = idx / (RT / 8), cv = idx % (RT / 8);
       *(uint4*)(Xs + j * XS + cv * 8) = xr[v];
+      if (do_n) {
+        const uint32_t in[4] = {xr[v].x, xr[v].y, xr[v].z, xr[v].w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          np[2 * p] += xsc[v] * __uint_as_float(in[p] << 16);
+          np[2 * p + 1] += xsc[v] * __uint_as_float(in[p] & 0xffff0000u);
+        }
+      }
+    }
+    if (do_n) {
+      // thread (row group tid/(RT/8), column vector tid%(RT/8)) holds the sum over its XV rows
+      float* dst = npart + (tid / (RT / 8)) * RT + (tid % (RT / 8)) * 8;
+      *(float4*)dst = make_float4(np[0], np[1], np[2], np[3]);
+      *(float4*)(dst + 4) = make_float4(np[4], np[5], np[6], np[7]);
     }
 #pragma unroll
     for (int v = 0; v < YV; ++v) {
@@ -113,13 +149,11 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       for (int p = 0; p < 4; ++p) {
         const float e0 = __uint_as_float(in[p] << 16) * ysc[v];
         const float e1 = __uint_as_float(in[p] & 0xffff0000u) * ysc[v];
-        const uint16_t h0 = f32_to_bf16_bits(e0), h1 = f32_to_bf16_bits(e1);
-        hi[p] = (uint32_t)h0 | ((uint32_t)h1 << 16);
-        if (HILO) lo[p] = pack_bf16x2(e0 - bf16_bits_to_f32(h0), e1 - bf16_bits_to_f32(h1));
+        hi[p] = pack_bf16x2(e0, e1);
+        if (HILO) lo[p] = pack_bf16x2(e0 - __uint_as_float(hi[p] << 16), e1 - __uint_as_float(hi[p] & 0xffff0000u));
       }
       *(uint4*)(Yh + j * YS + cv * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
       if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-      if (cv == 0) sc[j] = ysc[v];
     }
     __syncthreads();
     if (it + 1 < NC) prefetch(c + c_step);
@@ -181,11 +215,11 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
         }
     }
     // ---- normaliser vector (forward, first column tile only): n = gbar n + sum_j abar_j k_j
-    if (do_n) {
+    if (do_n && tid < RT) {
       a.nstates[((size_t)bh * NC + c) * DHQK + d_tile + tid] = nval;
       float s = 0.f;
-#pragma unroll 8
-      for (int j = 0; j < 128; ++j) s += sc[j] * bf16_bits_to_f32(Xs[j * XS + tid]);
+#pragma unroll
+      for (int g2 = 0; g2 < XROWS; ++g2) s += npart[g2 * RT + tid];
       nval = g * nval + s;
     }
     __syncthreads();
@@ -203,20 +237,17 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
           a.final_out[((size_t)bh * DHQK + d) * DHHV + w] = acc[db][wb][i];
         }
   }
-  if (do_n && a.n_final != nullptr) a.n_final[(size_t)bh * DHQK + d_tile + tid] = nval;
+  if (do_n && tid < RT && a.n_final != nullptr) a.n_final[(size_t)bh * DHQK + d_tile + tid] = nval;
 }
 
 template <int RT, int WT, bool HILO>
 static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
   constexpr int NT = 64 * (RT / 64) * (WT / 64);
-  const size_t smem = (size_t)128 * (RT + 16) * 2 + (size_t)128 * (WT + 16) * 2 * (HILO ? 2 : 1) + 128 * 4;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess)
-      return "scan: cannot raise the dynamic LDS limit";
-    attr_set = true;
-  }
+  constexpr int XROWS = NT / (RT / 8);
+  const size_t smem = (size_t)128 * (RT + 16) * 2 + (size_t)128 * (WT + 16) * 2 * (HILO ? 2 : 1) + (size_t)XROWS * RT * 4;
+  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)smem) != hipSuccess)
+    return "scan: cannot raise the dynamic LDS limit";
   dim3 grid(a.DHQK / RT, a.DHHV / WT, BH);
   hipLaunchKernelGGL((scan_kernel<RT, WT, HILO>), grid, dim3(NT), smem, stream, a);
   return nullptr;
