@@ -14,14 +14,19 @@
 // The state fragments (stored for a contraction over the head dimension) are copied to LDS unchanged and
 // re-read with the transposing LDS read, which hands out operands for a contraction over value columns.
 // Row sums  sum_d x[n][d] * Out[n][d]  (x = q for dQ, k for dK) are emitted for the gate gradients.
+//
+// A workgroup owns MT head-dim rows x 64 positions (half a chunk); every slab is fetched from global memory
+// into registers while the previous one is being multiplied, and the footprint (80 KB of LDS) lets two
+// workgroups share a CU so that one computes while the other waits for memory.
 #include "common.h"
 #include "kernels.h"
 
 namespace mlstm {
 
 template <int MT, bool IS_DQ>
-__global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
-  constexpr int MB = MT / 64;       // 32-row head-dim blocks per wave
+__global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
+  constexpr int NWAVE = MT / 64;    // each wave owns 64 head-dim rows = 2 MFMA row blocks
+  constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;       // P stored as Ps[n][o]
   constexpr int XS = 64 + 8;        // value-column slab row stride
   constexpr int ZS = MT + 16;       // pass-2 slab row stride
@@ -31,116 +36,152 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   // stage region: [state frags | Xn slab | Xo slab], later pass-2 slabs, later the output staging tile
-  constexpr int stage_elems_a = CF + 2 * 128 * XS;
-  constexpr int stage_elems_b = 128 * OS;
-  constexpr int stage_elems = stage_elems_a > stage_elems_b ? stage_elems_a : stage_elems_b;
+  constexpr int stage_elems_a = CF + 64 * XS + 128 * XS;
+  constexpr int stage_elems_b = 64 * OS;
+  constexpr int stage_elems_c = 32 * ZS;
+  constexpr int stage_ab = stage_elems_a > stage_elems_b ? stage_elems_a : stage_elems_b;
+  constexpr int stage_elems = stage_ab > stage_elems_c ? stage_ab : stage_elems_c;
   uint16_t* Cf = (uint16_t*)smem_raw;
   uint16_t* Xn = Cf + CF;
-  uint16_t* Xo = Xn + 128 * XS;
+  uint16_t* Xo = Xn + 64 * XS;
   uint16_t* Ps = Cf + stage_elems;
-  float* uu = (float*)(Ps + 128 * PS);
-  float* ww = uu + 128;
-  float* cs = ww + 128;    // column scale
-  float* rho = cs + 128;   // 1/(nrow + eps)
+  float* uu = (float*)(Ps + 64 * PS);  // [128]
+  float* ww = uu + 128;                // [128]
+  float* rho = ww + 128;               // [128] 1/(nrow + eps)
+  float* cs = rho + 128;               // [64] column scale of this workgroup's positions
+  float* red = cs + 64;                // [NWAVE][64] row-dot partials
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int mi = wave >> 1, ni = wave & 1;
   const int r = lane & 31, h = lane >> 5;
   const BlockId blk = xcd_block_id();
   const int bh = blk.z, c = blk.y;
-  const int d_tile = blk.x * MT;
+  const int nh = blk.x & 1;
+  const int d_tile = (blk.x >> 1) * MT;
   const size_t Sp = (size_t)NC * kChunk;
   const size_t gofs = bh * Sp + (size_t)c * kChunk;
   const int t_base = c * kChunk;
+  const int n0 = 64 * nh;
+  // live 32-row blocks of the other position index: dQ o = j <= t, dK o = t >= j
+  const int ob_lo = IS_DQ ? 0 : 2 * nh, ob_hi = IS_DQ ? 2 * (nh + 1) : 4;
   const uint16_t* Xn_g = (IS_DQ ? a.dH : a.V) + (size_t)bh * S * DHHV;
   const uint16_t* Xo_g = (IS_DQ ? a.V : a.dH) + (size_t)bh * S * DHHV;
   const uint16_t* Z_g = (IS_DQ ? a.K : a.Q) + (size_t)bh * S * DHQK + d_tile;
 
-  if (tid < 128) {
-    uu[tid] = a.g.u[gofs + tid];
-    ww[tid] = a.g.w[gofs + tid];
-    const float rh = a.use_nrow ? 1.f / (a.nrow[gofs + tid] + a.eps) : 1.f;
-    rho[tid] = rh;
-    cs[tid] = IS_DQ ? a.g.bbar[gofs + tid] * a.qk_scale * rh : a.g.abar[gofs + tid];
+  for (int idx = tid; idx < 128; idx += NTH) {
+    uu[idx] = a.g.u[gofs + idx];
+    ww[idx] = a.g.w[gofs + idx];
+    rho[idx] = a.use_nrow ? 1.f / (a.nrow[gofs + idx] + a.eps) : 1.f;
+  }
+  for (int idx = tid; idx < 64; idx += NTH) {
+    const float rh = a.use_nrow ? 1.f / (a.nrow[gofs + n0 + idx] + a.eps) : 1.f;
+    cs[idx] = IS_DQ ? a.g.bbar[gofs + n0 + idx] * a.qk_scale * rh : a.g.abar[gofs + n0 + idx];
   }
 
-  f32x16 acc[MB][2], sacc[2][2];
+  constexpr int OBW = (4 + NWAVE - 1) / NWAVE;  // score blocks per wave (at most)
+  f32x16 acc[2][2], sacc[OBW][2];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
+  for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
 #pragma unroll
-  for (int ob = 0; ob < 2; ++ob)
+  for (int k = 0; k < OBW; ++k)
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[ob][nb][i] = 0.f;
-  // dQ: o = j, n = t: dead quadrant j-half 1 / t-half 0.  dK: o = t, n = j: dead quadrant t-half 0 / j-half 1.
-  const bool quadrant_live = IS_DQ ? !(mi == 1 && ni == 0) : !(mi == 0 && ni == 1);
-  const int m_wave = mi * (MT / 2);
+      for (int i = 0; i < 16; ++i) sacc[k][nb][i] = 0.f;
+  const int m_wave = wave * 64;
 
-  // ---- pass 1 over the value columns
+  // ---- pass 1 over the value columns, 64 per slab, register-prefetched one slab ahead
   {
     const size_t ND = DHQK / 16, NW = DHHV / 32;
     const uint4* st = (const uint4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
+    constexpr int CV = 2 * NDT * 64 / NTH;  // state-fragment vectors per thread per slab
+    constexpr int NV = 64 * 8 / NTH;        // Xn vectors per thread per slab
+    constexpr int OV = 128 * 8 / NTH;       // Xo vectors per thread per slab
+    uint4 creg[CV], nreg[NV], oreg[OV];
+    auto load_slab = [&](int slab) {
+#pragma unroll
+      for (int v = 0; v < CV; ++v) {
+        const int idx = tid + v * NTH;
+        const int wb_l = idx / (NDT * 64), rem = idx % (NDT * 64);
+        creg[v] = st[((size_t)(2 * slab + wb_l) * ND + d_tile / 16) * 64 + rem];
+      }
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const int idx = tid + v * NTH;
+        const int j = idx >> 3, cv = idx & 7;
+        const int t = t_base + n0 + j;
+        nreg[v] = t < S ? *(const uint4*)(Xn_g + (size_t)t * DHHV + slab * 64 + cv * 8) : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < OV; ++v) {
+        const int idx = tid + v * NTH;
+        const int j = idx >> 3, cv = idx & 7;
+        const int t = t_base + j;
+        const bool live = j >= 32 * ob_lo && j < 32 * ob_hi && t < S;
+        oreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHHV + slab * 64 + cv * 8) : make_uint4(0, 0, 0, 0);
+      }
+    };
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     // transposing read of the staged fragments: lane i16 of a 16-lane block addresses value column
     // k0 + i16/4 and the 4 consecutive head-dim rows n0 + 4*(i16%4) .. +3
-    const int d_grp = i16 & 3;                          // which group of 4 rows inside the 16-row fragment
+    const int d_grp = i16 & 3;
     const int frag_byte = 32 * (d_grp & 1) * 16 + 8 * (d_grp >> 1);  // h_src = d_grp & 1, a_src = d_grp >> 1
-    for (int slab = 0; slab < DHHV / 64; ++slab) {
+    const int nslab = DHHV / 64;
+    load_slab(0);
+    for (int slab = 0; slab < nslab; ++slab) {
       __syncthreads();
-      // state fragments of value blocks 2*slab, 2*slab+1 and head-dim fragments of this tile: contiguous per block
-      for (int idx = tid; idx < 2 * NDT * 64; idx += 256) {
-        const int wb_l = idx / (NDT * 64), rem = idx % (NDT * 64);
-        ((uint4*)Cf)[idx] = st[((size_t)(2 * slab + wb_l) * ND + d_tile / 16) * 64 + rem];
+#pragma unroll
+      for (int v = 0; v < CV; ++v) ((uint4*)Cf)[tid + v * NTH] = creg[v];
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        const int idx = tid + v * NTH;
+        *(uint4*)(Xn + (idx >> 3) * XS + (idx & 7) * 8) = nreg[v];
       }
 #pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        const int idx = tid + v * 256;
-        const int j = idx >> 3, cv = idx & 7;
-        const int t = t_base + j;
-        const bool ok = t < S;
-        const size_t go = (size_t)t * DHHV + slab * 64 + cv * 8;
-        *(uint4*)(Xn + j * XS + cv * 8) = ok ? *(const uint4*)(Xn_g + go) : make_uint4(0, 0, 0, 0);
-        *(uint4*)(Xo + j * XS + cv * 8) = ok ? *(const uint4*)(Xo_g + go) : make_uint4(0, 0, 0, 0);
+      for (int v = 0; v < OV; ++v) {
+        const int idx = tid + v * NTH;
+        *(uint4*)(Xo + (idx >> 3) * XS + (idx & 7) * 8) = oreg[v];
       }
       __syncthreads();
+      if (slab + 1 < nslab) load_slab(slab + 1);
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         Frag B[2];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Xn + (64 * ni + 32 * nb + r) * XS + 16 * ks + 8 * h);
+        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Xn + (32 * nb + r) * XS + 16 * ks + 8 * h);
         // inter-chunk product: A = State[d][w]
         {
-          Frag A[MB];
-          const int wrow = 16 * ks + 8 * h + (i16 >> 2);      // value column inside the slab (first read)
+          Frag A[2];
+          const int wrow = 16 * ks + 8 * h + (i16 >> 2);  // value column inside the slab (first read)
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb) {
+          for (int mb = 0; mb < 2; ++mb) {
             const int ds_l = (m_wave + 32 * mb + 16 * q16) / 16;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
               const int wr = wrow + 4 * half;
-              const unsigned char* p = (const unsigned char*)Cf + ((size_t)((wr >> 5) * NDT + ds_l) * 64 + (wr & 31)) * 16 + frag_byte;
+              const unsigned char* p =
+                  (const unsigned char*)Cf + ((size_t)((wr >> 5) * NDT + ds_l) * 64 + (wr & 31)) * 16 + frag_byte;
               A[mb].d[half] = lds_read_tr16(p);
             }
           }
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
+          for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
         }
-        // score matrix: A = Xo rows
-        if (quadrant_live) {
-          Frag A[2];
+        // score matrix: A = Xo rows of the blocks dealt to this wave
 #pragma unroll
-          for (int ob = 0; ob < 2; ++ob) A[ob].u = *(const uint4*)(Xo + (64 * mi + 32 * ob + r) * XS + 16 * ks + 8 * h);
+        for (int k = 0; k < OBW; ++k) {
+          const int ob = ob_lo + wave + k * NWAVE;
+          if (ob < ob_hi) {
+            Frag A;
+            A.u = *(const uint4*)(Xo + (32 * ob + r) * XS + 16 * ks + 8 * h);
 #pragma unroll
-          for (int ob = 0; ob < 2; ++ob)
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb) mfma32(sacc[ob][nb], A[ob], B[nb]);
+            for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
+          }
         }
       }
     }
@@ -148,70 +189,85 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
   // column scale of the inter-chunk part
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const float sc = cs[64 * ni + 32 * nb + r];
+    const float sc = cs[32 * nb + r];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][nb] *= sc;
+    for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= sc;
   }
+  // first pass-2 slab into registers while the score matrix is gated
+  constexpr int ZV = 32 * (MT / 8) / NTH;
+  uint4 zreg[ZV];
+  auto load_zslab = [&](int ob) {
+#pragma unroll
+    for (int v = 0; v < ZV; ++v) {
+      const int idx = tid + v * NTH;
+      const int j = idx / (MT / 8), cv = idx % (MT / 8);
+      const int t = t_base + 32 * ob + j;
+      zreg[v] = t < S ? *(const uint4*)(Z_g + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  load_zslab(ob_lo);
   // gate the score matrix: P[o][n] = sacc * exp(u_t - w_j)/sqrt(DHQK) * rho_t for j <= t; store as Ps[n][o]
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const int n = 64 * ni + 32 * nb + r;
-    const float xn = IS_DQ ? uu[n] : ww[n];
-    const float rn = IS_DQ ? rho[n] : 1.f;
+  for (int k = 0; k < OBW; ++k) {
+    const int ob = ob_lo + wave + k * NWAVE;
+    if (ob < ob_hi) {
 #pragma unroll
-    for (int ob = 0; ob < 2; ++ob)
+      for (int nb = 0; nb < 2; ++nb) {
+        const int nl = 32 * nb + r;
+        const int n = n0 + nl;
+        const float xn = IS_DQ ? uu[n] : ww[n];
+        const float rn = IS_DQ ? rho[n] : 1.f;
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int o0 = 64 * mi + 32 * ob + 8 * g4 + 4 * h;
-        const float4 xo = *(const float4*)((IS_DQ ? ww : uu) + o0);
-        const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
-        float ro[4] = {1.f, 1.f, 1.f, 1.f};
-        if (!IS_DQ) {
-          const float4 rr = *(const float4*)(rho + o0);
-          ro[0] = rr.x; ro[1] = rr.y; ro[2] = rr.z; ro[3] = rr.w;
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int o0 = 32 * ob + 8 * g4 + 4 * h;
+          const float4 xo = *(const float4*)((IS_DQ ? ww : uu) + o0);
+          const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
+          float ro[4] = {1.f, 1.f, 1.f, 1.f};
+          if (!IS_DQ) {
+            const float4 rr = *(const float4*)(rho + o0);
+            ro[0] = rr.x; ro[1] = rr.y; ro[2] = rr.z; ro[3] = rr.w;
+          }
+          float pv[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float ex = IS_DQ ? (xn - xov[e]) : (xov[e] - xn);
+            const bool keep = IS_DQ ? (o0 + e <= n) : (n <= o0 + e);
+            const float val = sacc[k][nb][4 * g4 + e] * a.qk_scale * __expf(ex) * rn * ro[e];
+            pv[e] = keep ? val : 0.f;
+          }
+          *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
         }
-        float pv[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float ex = IS_DQ ? (xn - xov[e]) : (xov[e] - xn);
-          const bool keep = IS_DQ ? (o0 + e <= n) : (n <= o0 + e);
-          const float val = sacc[ob][nb][4 * g4 + e] * a.qk_scale * __expf(ex) * rn * ro[e];
-          pv[e] = keep ? val : 0.f;
-        }
-        *(uint2*)(Ps + n * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
       }
+    }
   }
 
-  // ---- pass 2 over the chunk positions o: Out^T += Z^T P
+  // ---- pass 2 over the live chunk positions o: Out^T += Z^T P
   {
     uint16_t* Zs = Cf;
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
-    for (int slab = 0; slab < 4; ++slab) {
+    for (int ob = ob_lo; ob < ob_hi; ++ob) {
       __syncthreads();  // first pass: P written and pass-1 slabs consumed
-      constexpr int vec_per_row = MT / 8;
-      for (int idx = tid; idx < 32 * vec_per_row; idx += 256) {
-        const int j = idx / vec_per_row, cv = idx % vec_per_row;
-        const int t = t_base + slab * 32 + j;
-        *(uint4*)(Zs + j * ZS + cv * 8) = t < S ? *(const uint4*)(Z_g + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < ZV; ++v) {
+        const int idx = tid + v * NTH;
+        *(uint4*)(Zs + (idx / (MT / 8)) * ZS + (idx % (MT / 8)) * 8) = zreg[v];
       }
       __syncthreads();
-      // dQ (n = t, o = j <= t): queries < 64 skip key slabs >= 2.  dK (n = j, o = t >= j): keys >= 64 skip query slabs < 2.
-      if (IS_DQ ? (ni == 0 && slab >= 2) : (ni == 1 && slab < 2)) continue;
+      if (ob + 1 < ob_hi) load_zslab(ob + 1);
 #pragma unroll
       for (int jl = 0; jl < 2; ++jl) {
-        Frag A[MB], B[2];
+        Frag A[2], B[2];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
+        for (int mb = 0; mb < 2; ++mb) {
           const uint16_t* p = Zs + (16 * jl + krow) * ZS + (m_wave + 32 * mb + ncol);
           A[mb].d[0] = lds_read_tr16(p);
           A[mb].d[1] = lds_read_tr16(p + 4 * ZS);
         }
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
-          B[nb].u = *(const uint4*)(Ps + (64 * ni + 32 * nb + r) * PS + slab * 32 + 16 * jl + 8 * h);
+        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + 32 * ob + 16 * jl + 8 * h);
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
           for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
       }
@@ -226,59 +282,60 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
   {
     const uint16_t* Rg = (IS_DQ ? a.Q : a.K) + (size_t)bh * S * DHQK + d_tile;
     constexpr int vec_per_row = MT / 8;
-    for (int idx = tid; idx < 128 * vec_per_row; idx += 256) {
+    for (int idx = tid; idx < 64 * vec_per_row; idx += NTH) {
       const int j = idx / vec_per_row, cv = idx % vec_per_row;
-      const int t = t_base + j;
+      const int t = t_base + n0 + j;
       *(uint4*)(Os + j * OS + cv * 8) = t < S ? *(const uint4*)(Rg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
     }
   }
   __syncthreads();
-  float* red = uu;  // [2][128]: uu/ww are dead after the gating step
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const int n = 64 * ni + 32 * nb + r;
+    const int nl = 32 * nb + r;
     float part = 0.f;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int d0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
-        const uint2 xv = *(const uint2*)(Os + n * OS + d0);
+        const uint2 xv = *(const uint2*)(Os + nl * OS + d0);
         part += acc[mb][nb][4 * g4 + 0] * __uint_as_float(xv.x << 16);
         part += acc[mb][nb][4 * g4 + 1] * __uint_as_float(xv.x & 0xffff0000u);
         part += acc[mb][nb][4 * g4 + 2] * __uint_as_float(xv.y << 16);
         part += acc[mb][nb][4 * g4 + 3] * __uint_as_float(xv.y & 0xffff0000u);
       }
     part += __shfl_xor(part, 32);
-    if (h == 0) red[mi * 128 + n] = part;
+    if (h == 0) red[wave * 64 + nl] = part;
   }
   __syncthreads();
-  if (tid < 128) {
-    const float dot = red[tid] + red[128 + tid];
-    if (gridDim.x == 1) a.rowdot[gofs + tid] = dot;
-    else atomicAdd(a.rowdot + gofs + tid, dot);
+  if (tid < 64) {
+    float dot = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWAVE; ++w) dot += red[w * 64 + tid];
+    if (gridDim.x == 2) a.rowdot[gofs + n0 + tid] = dot;
+    else atomicAdd(a.rowdot + gofs + n0 + tid, dot);
   }
 
   // ---- epilogue part 2: round, transpose through LDS, coalesced store
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const int n = 64 * ni + 32 * nb + r;
+    const int nl = 32 * nb + r;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int d0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
-        *(uint2*)(Os + n * OS + d0) = make_uint2(pack_bf16x2(acc[mb][nb][4 * g4 + 0], acc[mb][nb][4 * g4 + 1]),
-                                                 pack_bf16x2(acc[mb][nb][4 * g4 + 2], acc[mb][nb][4 * g4 + 3]));
+        *(uint2*)(Os + nl * OS + d0) = make_uint2(pack_bf16x2(acc[mb][nb][4 * g4 + 0], acc[mb][nb][4 * g4 + 1]),
+                                                  pack_bf16x2(acc[mb][nb][4 * g4 + 2], acc[mb][nb][4 * g4 + 3]));
       }
   }
   __syncthreads();
   {
     uint16_t* Og = a.Out + (size_t)bh * S * DHQK + d_tile;
     constexpr int vec_per_row = MT / 8;
-    for (int idx = tid; idx < 128 * vec_per_row; idx += 256) {
+    for (int idx = tid; idx < 64 * vec_per_row; idx += NTH) {
       const int j = idx / vec_per_row, cv = idx % vec_per_row;
-      const int t = t_base + j;
+      const int t = t_base + n0 + j;
       if (t < S) *(uint4*)(Og + (size_t)t * DHQK + cv * 8) = *(const uint4*)(Os + j * OS + cv * 8);
     }
   }
@@ -287,13 +344,15 @@ __global__ __launch_bounds__(256) void par_qk_kernel(ParQkArgs a) {
 template <int MT, bool IS_DQ>
 static const char* launch_par_qk_t(const ParQkArgs& a, int BH, hipStream_t stream) {
   constexpr int CF = 2 * (MT / 16) * 64 * 8;
-  constexpr int sa = CF + 2 * 128 * 72, sb = 128 * (MT + 8);
-  const size_t smem = (size_t)((sa > sb ? sa : sb) + 128 * 136) * 2 + 4 * 128 * 4;
+  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
+  constexpr int sab = sa > sb ? sa : sb;
+  constexpr int stage = sab > sc ? sab : sc;
+  const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;
   if (hipFuncSetAttribute((const void*)par_qk_kernel<MT, IS_DQ>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_qk: cannot raise the dynamic LDS limit";
-  dim3 grid(a.DHQK / MT, a.NC, BH);
-  hipLaunchKernelGGL((par_qk_kernel<MT, IS_DQ>), grid, dim3(256), smem, stream, a);
+  dim3 grid(2 * (a.DHQK / MT), a.NC, BH);
+  hipLaunchKernelGGL((par_qk_kernel<MT, IS_DQ>), grid, dim3(MT), smem, stream, a);
   return nullptr;
 }
 

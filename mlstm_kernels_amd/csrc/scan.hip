@@ -84,16 +84,9 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   const uint16_t* Yg = a.Y + (size_t)bh * S * DHHV + w_tile;
 
   uint4 xr[XV], yr[YV];
-  float xsc[XV], ysc[YV];
-  auto row_scale = [&](int t) -> float {
-    if (t >= S) return 0.f;
-    float s = a.scale_a[bh * Sp + t];
-    if (a.backward) {
-      s *= a.qk_scale;
-      if (a.nrow != nullptr) s /= (a.nrow[bh * Sp + t] + a.eps);
-    }
-    return s;
-  };
+  float xsc[XV], ysc[YV], ynr[YV];
+  // The prefetch only LOADS (raw scale factors included): any arithmetic on a loaded value here would make the
+  // wave wait for the whole batch of loads before it starts the matrix work they are meant to overlap with.
   auto prefetch = [&](int c) {
 #pragma unroll
     for (int v = 0; v < XV; ++v) {
@@ -101,7 +94,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       const int j = idx / (RT / 8), cv = idx % (RT / 8);
       const int t = c * kChunk + j;
       xr[v] = t < S ? *(const uint4*)(Xg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
-      if (do_n) xsc[v] = row_scale(t);
+      if (do_n) xsc[v] = t < S ? a.scale_a[bh * Sp + t] : 0.f;
     }
 #pragma unroll
     for (int v = 0; v < YV; ++v) {
@@ -109,7 +102,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
       const int t = c * kChunk + j;
       yr[v] = t < S ? *(const uint4*)(Yg + (size_t)t * DHHV + cv * 8) : make_uint4(0, 0, 0, 0);
-      ysc[v] = row_scale(t);
+      ysc[v] = t < S ? a.scale_a[bh * Sp + t] : 0.f;
+      if (a.backward && a.nrow != nullptr) ynr[v] = a.nrow[bh * Sp + t];
     }
   };
 
@@ -145,10 +139,15 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
       const uint32_t in[4] = {yr[v].x, yr[v].y, yr[v].z, yr[v].w};
       uint32_t hi[4], lo[4];
+      float sc = ysc[v];
+      if (a.backward) {
+        sc *= a.qk_scale;
+        if (a.nrow != nullptr) sc /= (ynr[v] + a.eps);
+      }
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const float e0 = __uint_as_float(in[p] << 16) * ysc[v];
-        const float e1 = __uint_as_float(in[p] & 0xffff0000u) * ysc[v];
+        const float e0 = __uint_as_float(in[p] << 16) * sc;
+        const float e1 = __uint_as_float(in[p] & 0xffff0000u) * sc;
         hi[p] = pack_bf16x2(e0, e1);
         if (HILO) lo[p] = pack_bf16x2(e0 - __uint_as_float(hi[p] << 16), e1 - __uint_as_float(hi[p] & 0xffff0000u));
       }

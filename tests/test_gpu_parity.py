@@ -98,7 +98,7 @@ def test_decode_after_prefill():
     dict(B=2, NH=4, S=512, DQK=128, DHV=256, L=256, seed=1, dtype=torch.bfloat16),  # BASELINE config 2
     dict(B=1, NH=2, S=144, DQK=64, DHV=128, L=16, seed=2, dtype=torch.bfloat16),   # ragged tail (128 + 16)
     dict(B=1, NH=2, S=32, DQK=64, DHV=64, L=32, seed=3, dtype=torch.bfloat16),     # shorter than one chunk
-    dict(B=1, NH=1, S=256, DQK=256, DHV=1024, L=128, seed=4, dtype=torch.bfloat16),  # several value-column tiles
+    dict(B=1, NH=1, S=256, DQK=512, DHV=1024, L=128, seed=4, dtype=torch.bfloat16),  # several head-dim / value tiles
 ])
 def test_chunkwise_forward_exp(cfg):
     exp_op, *_ = _ops()
@@ -129,7 +129,7 @@ def test_chunkwise_forward_gate_regimes(f_offset):
 
 def test_unsupported_head_dim_fails_loudly():
     exp_op, *_ = _ops()
-    q, k, v, i, f = make_qkvif(1, 1, 128, 512, 128)
+    q, k, v, i, f = make_qkvif(1, 1, 128, 1024, 128)
     with pytest.raises(RuntimeError, match="DHQK too large"):
         exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128)
     q, k, v, i, f = make_qkvif(1, 1, 128, 96, 128)
@@ -186,6 +186,7 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     dict(B=1, NH=2, S=256, DQK=64, DHV=128),
     dict(B=2, NH=2, S=512, DQK=128, DHV=256, seed=1),
     dict(B=1, NH=2, S=384, DQK=256, DHV=512, init=True, dcl=True),
+    dict(B=1, NH=1, S=256, DQK=512, DHV=256, init=True),          # two head-dim tiles: atomic row dots
     dict(B=1, NH=2, S=256, DQK=64, DHV=128, siging=True, init=True),
     dict(B=1, NH=2, S=256, DQK=64, DHV=64, siging=True, normalize=False),
     dict(B=1, NH=2, S=144, DQK=64, DHV=64, L=16),                  # ragged tail
