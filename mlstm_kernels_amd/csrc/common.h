@@ -13,6 +13,9 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+// 16 raw bytes as a native vector: unlike HIP's uint4 struct, a memory-to-memory copy through an array of these
+// is promoted to registers (struct copies become memcpy calls the optimiser leaves in scratch memory)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // 8 bf16 as raw bits; convertible to the MFMA operand type without data movement
 union Frag {

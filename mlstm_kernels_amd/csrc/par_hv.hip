@@ -53,7 +53,8 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   float* rows = inv + 128;              // [NWAVE][64] partial row sums of Sbar (forward)
   float* nperm = rows + NWAVE * 64;     // [DHQK] n_prev in fragment order (forward)
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
   const BlockId blk = xcd_block_id();  // halves and column tiles of one chunk share operands: same XCD
   const int bh = blk.z, c = blk.y;
@@ -123,17 +124,19 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
     if (slab + 1 < nslab) load_kslab(slab + 1);
 #pragma unroll
     for (int k = 0; k < OBW; ++k) {
+      // unconditional on purpose: a wave whose block lies above the diagonal multiplies zero rows (its result is
+      // dropped at the gating step); a branch here would make the compiler shuttle the score accumulators between
+      // the two register files on every iteration
       const int ob = ob_lo + wave + k * NWAVE;
-      if (ob < ob_hi) {
+      const int obc = ob < 4 ? ob : 3;
 #pragma unroll
-        for (int ds = 0; ds < 4; ++ds) {
-          Frag A, B[2];
-          A.u = *(const uint4*)(Ts + (32 * ob + r) * KS + 16 * ds + 8 * h);
+      for (int ds = 0; ds < 4; ++ds) {
+        Frag A, B[2];
+        A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
+        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
-        }
+        for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
       }
     }
   }

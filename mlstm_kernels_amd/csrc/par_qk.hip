@@ -28,11 +28,11 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
   constexpr int NWAVE = MT / 64;    // each wave owns 64 head-dim rows = 2 MFMA row blocks
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;       // P stored as Ps[n][o]
-  constexpr int XS = 64 + 8;        // value-column slab row stride
+  constexpr int XS = 32 + 8;        // value-column slab row stride (32 columns per slab)
   constexpr int ZS = MT + 16;       // pass-2 slab row stride
   constexpr int OS = MT + 8;        // output staging row stride
   constexpr int NDT = MT / 16;      // 16-row state fragments per 32 value columns inside the tile
-  constexpr int CF = 2 * NDT * 64 * 8;  // elements of the staged state fragments per 64-column slab
+  constexpr int CF = NDT * 64 * 8;  // elements of the staged state fragments per 32-column slab
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   // stage region: [state frags | Xn slab | Xo slab], later pass-2 slabs, later the output staging tile
@@ -51,7 +51,8 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
   float* cs = rho + 128;               // [64] column scale of this workgroup's positions
   float* red = cs + 64;                // [NWAVE][64] row-dot partials
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
   const BlockId blk = xcd_block_id();
   const int bh = blk.z, c = blk.y;
@@ -93,62 +94,65 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
       for (int i = 0; i < 16; ++i) sacc[k][nb][i] = 0.f;
   const int m_wave = wave * 64;
 
-  // ---- pass 1 over the value columns, 64 per slab, register-prefetched one slab ahead
+  // ---- pass 1 over the value columns, 32 per slab, register-prefetched one slab ahead
   {
     const size_t ND = DHQK / 16, NW = DHHV / 32;
-    const uint4* st = (const uint4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
-    constexpr int CV = 2 * NDT * 64 / NTH;  // state-fragment vectors per thread per slab
-    constexpr int NV = 64 * 8 / NTH;        // Xn vectors per thread per slab
-    constexpr int OV = 128 * 8 / NTH;       // Xo vectors per thread per slab
-    uint4 creg[CV], nreg[NV], oreg[OV];
-    auto load_slab = [&](int slab) {
-#pragma unroll
-      for (int v = 0; v < CV; ++v) {
-        const int idx = tid + v * NTH;
-        const int wb_l = idx / (NDT * 64), rem = idx % (NDT * 64);
-        creg[v] = st[((size_t)(2 * slab + wb_l) * ND + d_tile / 16) * 64 + rem];
-      }
-#pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        const int idx = tid + v * NTH;
-        const int j = idx >> 3, cv = idx & 7;
-        const int t = t_base + n0 + j;
-        nreg[v] = t < S ? *(const uint4*)(Xn_g + (size_t)t * DHHV + slab * 64 + cv * 8) : make_uint4(0, 0, 0, 0);
-      }
-#pragma unroll
-      for (int v = 0; v < OV; ++v) {
-        const int idx = tid + v * NTH;
-        const int j = idx >> 3, cv = idx & 7;
-        const int t = t_base + j;
-        const bool live = j >= 32 * ob_lo && j < 32 * ob_hi && t < S;
-        oreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHHV + slab * 64 + cv * 8) : make_uint4(0, 0, 0, 0);
-      }
-    };
+    const u32x4* st = (const u32x4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
+    constexpr int CV = NDT * 64 / NTH;      // state-fragment vectors per thread per slab
+    constexpr int NV = 64 * 4 / NTH;        // Xn vectors per thread per slab
+    constexpr int OV = 128 * 4 / NTH;       // Xo vectors per thread per slab
+    u32x4 creg[CV];
+    uint4 nreg[NV], oreg[OV];
+    // (a macro, not a lambda: with the arrays captured by reference the compiler kept them in scratch memory)
+#define MLSTM_LOAD_SLAB(slab_)                                                                                       \
+  {                                                                                                                  \
+    _Pragma("unroll") for (int v = 0; v < CV; ++v)                                                                   \
+        creg[v] = st[((size_t)(slab_) * ND + d_tile / 16) * 64 + tid + v * NTH];                                     \
+    _Pragma("unroll") for (int v = 0; v < NV; ++v) {                                                                 \
+      const int idx = tid + v * NTH;                                                                                 \
+      const int t = t_base + n0 + (idx >> 2);                                                                        \
+      nreg[v] = t < S ? *(const uint4*)(Xn_g + (size_t)t * DHHV + (slab_) * 32 + (idx & 3) * 8) : make_uint4(0, 0, 0, 0); \
+    }                                                                                                                \
+    _Pragma("unroll") for (int v = 0; v < OV; ++v) {                                                                 \
+      const int idx = tid + v * NTH;                                                                                 \
+      const int j = idx >> 2;                                                                                        \
+      const int t = t_base + j;                                                                                      \
+      const bool live = j >= 32 * ob_lo && j < 32 * ob_hi && t < S;                                                  \
+      oreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHHV + (slab_) * 32 + (idx & 3) * 8) : make_uint4(0, 0, 0, 0); \
+    }                                                                                                                \
+  }
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     // transposing read of the staged fragments: lane i16 of a 16-lane block addresses value column
     // k0 + i16/4 and the 4 consecutive head-dim rows n0 + 4*(i16%4) .. +3
     const int d_grp = i16 & 3;
-    const int frag_byte = 32 * (d_grp & 1) * 16 + 8 * (d_grp >> 1);  // h_src = d_grp & 1, a_src = d_grp >> 1
-    const int nslab = DHHV / 64;
-    load_slab(0);
+    const int h_src = d_grp & 1, a_src = d_grp >> 1;
+    const int nslab = DHHV / 32;
+    MLSTM_LOAD_SLAB(0)
     for (int slab = 0; slab < nslab; ++slab) {
       __syncthreads();
 #pragma unroll
-      for (int v = 0; v < CV; ++v) ((uint4*)Cf)[tid + v * NTH] = creg[v];
+      for (int v = 0; v < CV; ++v) {
+        // lanes 32..63 of every fragment are stored 4 slots off so that the two lane halves a transposing read
+        // touches together fall on different LDS banks
+        const int idx = tid + v * NTH;
+        ((u32x4*)Cf)[idx ^ (((idx >> 5) & 1) << 2)] = creg[v];
+      }
 #pragma unroll
       for (int v = 0; v < NV; ++v) {
         const int idx = tid + v * NTH;
-        *(uint4*)(Xn + (idx >> 3) * XS + (idx & 7) * 8) = nreg[v];
+        *(uint4*)(Xn + (idx >> 2) * XS + (idx & 3) * 8) = nreg[v];
       }
 #pragma unroll
       for (int v = 0; v < OV; ++v) {
         const int idx = tid + v * NTH;
-        *(uint4*)(Xo + (idx >> 3) * XS + (idx & 7) * 8) = oreg[v];
+        *(uint4*)(Xo + (idx >> 2) * XS + (idx & 3) * 8) = oreg[v];
       }
       __syncthreads();
-      if (slab + 1 < nslab) load_slab(slab + 1);
+      // unconditional (the last iteration re-fetches its own slab): a conditional prefetch makes the compiler
+      // keep the prefetch registers in scratch memory across the loop back-edge
+      MLSTM_LOAD_SLAB(slab + 1 < nslab ? slab + 1 : slab)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
+      for (int ks = 0; ks < 2; ++ks) {
         Frag B[2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Xn + (32 * nb + r) * XS + 16 * ks + 8 * h);
@@ -162,8 +166,8 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
               const int wr = wrow + 4 * half;
-              const unsigned char* p =
-                  (const unsigned char*)Cf + ((size_t)((wr >> 5) * NDT + ds_l) * 64 + (wr & 31)) * 16 + frag_byte;
+              const int slot = (32 * h_src + wr) ^ (h_src << 2);
+              const unsigned char* p = (const unsigned char*)Cf + ((size_t)ds_l * 64 + slot) * 16 + 8 * a_src;
               A[mb].d[half] = lds_read_tr16(p);
             }
           }
@@ -175,17 +179,20 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
         // score matrix: A = Xo rows of the blocks dealt to this wave
 #pragma unroll
         for (int k = 0; k < OBW; ++k) {
+          // unconditional on purpose: a wave whose block lies above the diagonal multiplies zero rows (its result
+          // is dropped at the gating step); a branch here would make the compiler shuttle the score accumulators
+          // between the two register files on every iteration
           const int ob = ob_lo + wave + k * NWAVE;
-          if (ob < ob_hi) {
-            Frag A;
-            A.u = *(const uint4*)(Xo + (32 * ob + r) * XS + 16 * ks + 8 * h);
+          const int obc = ob < 4 ? ob : 3;
+          Frag A;
+          A.u = *(const uint4*)(Xo + (32 * obc + r) * XS + 16 * ks + 8 * h);
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
-          }
+          for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
         }
       }
     }
   }
+#undef MLSTM_LOAD_SLAB
   // column scale of the inter-chunk part
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
@@ -343,8 +350,8 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
 
 template <int MT, bool IS_DQ>
 static const char* launch_par_qk_t(const ParQkArgs& a, int BH, hipStream_t stream) {
-  constexpr int CF = 2 * (MT / 16) * 64 * 8;
-  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
+  constexpr int CF = (MT / 16) * 64 * 8;
+  constexpr int sa = CF + 64 * 40 + 128 * 40, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
   constexpr int sab = sa > sb ? sa : sb;
   constexpr int stage = sab > sc ? sab : sc;
   const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;

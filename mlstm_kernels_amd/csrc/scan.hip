@@ -39,7 +39,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   uint16_t* Yl = Yh + 128 * YS;
   float* npart = (float*)(Yl + (HILO ? 128 * YS : 0));  // [XROWS][RT] partial sums of the n update
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wr = wave / WC, wc = wave % WC;
   const int r = lane & 31, h = lane >> 5;
   // ---- XCD-aware renumbering: linear id -> (xcd, slot) -> contiguous range of ids per XCD
