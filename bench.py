@@ -42,9 +42,12 @@ FLOPS_PER_TOKEN_HEAD = {
     "par_dq": 2 * DHQK * DHHV + CHUNK * (DHHV + DHQK),  # dH C^T, causal dH V^T and dS K
     "par_dk": 2 * DHQK * DHHV + CHUNK * DHQK,           # V dC^T, causal dS^T Q
 }
+# the fused sequential kernels do the work of a scan plus the chunk-parallel kernel that follows it
+FLOPS_PER_TOKEN_HEAD["fused_fw"] = FLOPS_PER_TOKEN_HEAD["scan_fw"] + FLOPS_PER_TOKEN_HEAD["par_h"]
+FLOPS_PER_TOKEN_HEAD["fused_dv"] = FLOPS_PER_TOKEN_HEAD["scan_bw"] + FLOPS_PER_TOKEN_HEAD["par_dv"]
 FLOPS_FW = 4 * DHQK * DHHV + CHUNK * (DHQK + DHHV)
 FLOPS_BW = 8 * DHQK * DHHV + CHUNK * (3 * DHQK + 2 * DHHV)
-assert sum(FLOPS_PER_TOKEN_HEAD.values()) == FLOPS_FW + FLOPS_BW
+assert sum(FLOPS_PER_TOKEN_HEAD[n] for n in ("fused_fw", "fused_dv", "par_dq", "par_dk")) == FLOPS_FW + FLOPS_BW
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # decode step: bytes per (batch, head): C and n read+write fp32, m read+write, q,k,v in, h out (bf16), i,f

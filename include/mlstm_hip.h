@@ -48,6 +48,22 @@ int mlstm_hip_profile_read(int index, char* name, size_t name_cap, float* total_
 const char* mlstm_hip_last_error(void);
 
 /*
+ * Kernel selection for the value-column side of the chunkwise passes (H forward, dV backward).  A tuning knob with
+ * no counterpart in the reference (its Triton kernels are always the two-kernel form, recurrent_fw_C followed by
+ * parallel_fw_Hintra: mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:20-136).
+ *   MLSTM_PATH_AUTO  : the faster one for the shape as measured on MI355X (today: split for every shape)
+ *   MLSTM_PATH_SPLIT : state scan + chunk-parallel kernel over materialised chunk states
+ *   MLSTM_PATH_FUSED : one sequential kernel per pass, state slice resident in registers (falls back to split
+ *                      for head dimensions it does not support)
+ * Process-wide; returns the previous setting.  Results of the two paths agree within the rounding of bf16 operands.
+ * A forward workspace sized under one setting must be used under the same setting.
+ */
+#define MLSTM_PATH_AUTO 0
+#define MLSTM_PATH_SPLIT 1
+#define MLSTM_PATH_FUSED 2
+int mlstm_hip_set_chunkwise_path(int path);
+
+/*
  * Fused recurrent decode step (one token for every (b, head)).
  * Replaces: mlstm_kernels/torch/recurrent/triton_step.py:15-127 (mlstm_recurrent_step__triton_fw) and the
  * Triton kernel mlstm_kernels/triton/recurrent/fw_step_fused.py:19-195.

@@ -11,6 +11,7 @@ _lib = None
 
 F32, BF16 = 0, 1
 GATE_EXP, GATE_SIG = 0, 1
+PATH_AUTO, PATH_SPLIT, PATH_FUSED = 0, 1, 2
 ABI_VERSION = 1
 
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
@@ -19,6 +20,7 @@ _SIGNATURES = {
     "mlstm_hip_abi_version": (_i, []),
     "mlstm_hip_last_error": (ctypes.c_char_p, []),
     "mlstm_hip_profile_enable": (_i, [_i]),
+    "mlstm_hip_set_chunkwise_path": (_i, [_i]),
     "mlstm_hip_profile_read": (_i, [_i, ctypes.c_char_p, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)]),
     "mlstm_hip_step": (_i, [_vp] * 12 + [_i, _i, _i, _i, _f, _i, _i, _vp]),
     "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 6),
@@ -59,6 +61,11 @@ def get_lib() -> ctypes.CDLL:
                 )
             _lib = lib
     return _lib
+
+
+def set_chunkwise_path(path: int) -> int:
+    """Select the kernels of the chunkwise passes (PATH_AUTO / PATH_SPLIT / PATH_FUSED); returns the previous setting."""
+    return get_lib().mlstm_hip_set_chunkwise_path(int(path))
 
 
 def profile_enable(on: bool) -> None:

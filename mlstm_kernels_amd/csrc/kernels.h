@@ -42,6 +42,28 @@ struct ParHvArgs {
   int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant
 };
 
+struct FusedHvArgs {
+  const uint16_t *Q, *K, *V, *dH;  // forward uses Q,K,V; dV uses Q,K,dH
+  GateBufs g;
+  const float* init;        // (B,NH,DHQK,DHHV) fp32 initial state (forward: C0, dV: dC_last) or nullptr (zeros)
+  const float* n_init;      // forward: (B,NH,DHQK) or nullptr
+  const float* nrow;        // dV: row normaliser of the forward pass
+  uint16_t* states;         // bf16 state fragments [BH][NC][DHHV/32][DHQK/16][64][8] or nullptr (not emitted)
+  uint16_t* Out;            // (B,NH,S,DHHV) bf16: H or dV
+  float* nrow_out;          // forward: row normaliser (workspace [BH][Sp])
+  float* n_out;             // forward, optional (B,NH,S)
+  float* m_out;             // forward, optional (B,NH,S)
+  float* final_out;         // (B,NH,DHQK,DHHV) fp32 or nullptr: C_last (forward) / dC0 (dV)
+  float* n_final;           // forward: (B,NH,DHQK) or nullptr
+  int S, NC, DHQK, DHHV;
+  float qk_scale, eps;
+  int sig_gate;
+  int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant (n is then not tracked)
+#ifdef MLSTM_FUSED_TIMING
+  unsigned long long* timing;  // one-off timing builds: per-wave cycle counts of the phases of workgroup (0,0)
+#endif
+};
+
 struct ParQkArgs {
   const uint16_t *Q, *K, *V, *dH;
   GateBufs g;
@@ -69,6 +91,8 @@ const char* launch_gates(const void* i, const void* f, const float* m0, const Ga
                          int B, int NH, int S, int dtype_gates, int sig_gate, hipStream_t stream);
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream);
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream);
+bool fused_hv_supported(int DHQK, int DHHV);
+const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 const char* launch_par_qk(const ParQkArgs& a, int BH, bool is_dq, hipStream_t stream);
 const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream);
 const char* launch_fill_zero(float* p, size_t n, hipStream_t stream);

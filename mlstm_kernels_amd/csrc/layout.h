@@ -41,7 +41,8 @@ struct BwWorkspace {
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK, int DHHV) {
+// with_states = false leaves out the chunk states (forward passes whose states nobody reads: cstates is null)
+inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK, int DHHV, bool with_states) {
   const size_t BH = (size_t)B * NH, NC = (size_t)(S + 127) / 128, Sp = NC * 128;
   char* p = (char*)base;
   size_t off = 0;
@@ -61,7 +62,7 @@ inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK
   w.g.mstates = (float*)take(BH * (NC + 1) * 4);
   w.nstates = (float*)take(BH * NC * DHQK * 4);
   w.nrow = (float*)take(BH * Sp * 4);
-  w.cstates = (uint16_t*)take(BH * NC * (size_t)DHQK * DHHV * 2);
+  w.cstates = with_states ? (uint16_t*)take(BH * NC * (size_t)DHQK * DHHV * 2) : nullptr;
   w.bytes = off;
   return w;
 }

@@ -20,6 +20,17 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
+@pytest.fixture(autouse=True, params=["split", "fused"])
+def chunkwise_path(request):
+    """Every test runs once per kernel path of the chunkwise passes: 'split' (state scan + chunk-parallel kernels)
+    and 'fused' (sequential kernels with register-resident state; head dimensions they do not support fall back)."""
+    from mlstm_kernels_amd import _lib
+
+    previous = _lib.set_chunkwise_path(_lib.PATH_SPLIT if request.param == "split" else _lib.PATH_FUSED)
+    yield request.param
+    _lib.set_chunkwise_path(previous)
+
+
 def _ops():
     from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk
     from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_sequence__hip, mlstm_recurrent_step__hip
@@ -99,6 +110,9 @@ def test_decode_after_prefill():
     dict(B=1, NH=2, S=144, DQK=64, DHV=128, L=16, seed=2, dtype=torch.bfloat16),   # ragged tail (128 + 16)
     dict(B=1, NH=2, S=32, DQK=64, DHV=64, L=32, seed=3, dtype=torch.bfloat16),     # shorter than one chunk
     dict(B=1, NH=1, S=256, DQK=512, DHV=1024, L=128, seed=4, dtype=torch.bfloat16),  # several head-dim / value tiles
+    dict(B=1, NH=2, S=400, DQK=128, DHV=128, L=16, seed=5, dtype=torch.bfloat16),  # ragged tail (3 * 128 + 16)
+    dict(B=1, NH=1, S=32, DQK=256, DHV=64, L=32, seed=6, dtype=torch.bfloat16),    # shorter than one chunk
+    dict(B=2, NH=2, S=1024, DQK=256, DHV=192, L=128, seed=7, dtype=torch.bfloat16),  # three value slices
 ])
 def test_chunkwise_forward_exp(cfg):
     exp_op, *_ = _ops()
@@ -116,10 +130,11 @@ def test_chunkwise_forward_exp(cfg):
     assert torch.equal(H2, H)
 
 
+@pytest.mark.parametrize("DQK", [64, 128])
 @pytest.mark.parametrize("f_offset", [0.0, -3.0, 6.0])
-def test_chunkwise_forward_gate_regimes(f_offset):
+def test_chunkwise_forward_gate_regimes(f_offset, DQK):
     exp_op, *_ = _ops()
-    q, k, v, i, f = make_qkvif(1, 2, 384, 64, 128, seed=7, f_offset=f_offset)
+    q, k, v, i, f = make_qkvif(1, 2, 384, DQK, 128, seed=7, f_offset=f_offset)
     ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=64)
     H, (C, n, m) = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
     check_matrix(H, ref["H"], "H", frac=2e-3)
@@ -190,6 +205,9 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     dict(B=1, NH=2, S=256, DQK=64, DHV=128, siging=True, init=True),
     dict(B=1, NH=2, S=256, DQK=64, DHV=64, siging=True, normalize=False),
     dict(B=1, NH=2, S=144, DQK=64, DHV=64, L=16),                  # ragged tail
+    dict(B=1, NH=2, S=400, DQK=128, DHV=64, L=16, init=True, dcl=True, seed=2),   # ragged tail, initial state
+    dict(B=1, NH=2, S=256, DQK=128, DHV=128, siging=True, init=True, seed=3),
+    dict(B=1, NH=2, S=256, DQK=256, DHV=64, siging=True, normalize=False, seed=4),
 ])
 def test_chunkwise_fwbw_small(kw):
     _fwbw_case(**kw)
