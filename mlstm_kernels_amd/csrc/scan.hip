@@ -24,6 +24,8 @@
 
 namespace mlstm {
 
+constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in LDS
+
 template <int RT, int WT, bool HILO>
 __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanArgs a) {
   constexpr int WC = WT / 64;
@@ -38,6 +40,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   uint16_t* Yh = Xs + 128 * XS;
   uint16_t* Yl = Yh + 128 * YS;
   float* npart = (float*)(Yl + (HILO ? 128 * YS : 0));  // [XROWS][RT] partial sums of the n update
+  float* gl = npart + XROWS * RT;                       // [kGBlock] decay factors of the next chunks, in scan order
 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,6 +115,14 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   prefetch(c_first);
   for (int it = 0; it < NC; ++it) {
     const int c = c_first + it * c_step;
+    // The decay factors come from LDS, a block of chunks at a time: read straight from global memory inside the
+    // loop, the factor would sit behind the prefetch of the next chunk (loads complete in order) and the matrix
+    // work would wait for the whole prefetch in every iteration.
+    if ((it & (kGBlock - 1)) == 0) {
+      __syncthreads();
+      for (int k = tid; k < kGBlock && it + k < NC; k += NT) gl[k] = a.gbar[(size_t)bh * NC + c + k * c_step];
+      // visible after the barrier that follows the staging below
+    }
     // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split); partial sums of sum_j abar_j k_j
     float np[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -179,7 +190,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
         }
     }
     // ---- decay, then accumulate X^T (scale . Y) over the 128 positions of the chunk
-    const float g = a.gbar[(size_t)bh * NC + c];
+    const float g = gl[it & (kGBlock - 1)];
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -244,7 +255,8 @@ template <int RT, int WT, bool HILO>
 static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
   constexpr int NT = 64 * (RT / 64) * (WT / 64);
   constexpr int XROWS = NT / (RT / 8);
-  const size_t smem = (size_t)128 * (RT + 16) * 2 + (size_t)128 * (WT + 16) * 2 * (HILO ? 2 : 1) + (size_t)XROWS * RT * 4;
+  const size_t smem = (size_t)128 * (RT + 16) * 2 + (size_t)128 * (WT + 16) * 2 * (HILO ? 2 : 1) +
+                      (size_t)(XROWS * RT + kGBlock) * 4;
   if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "scan: cannot raise the dynamic LDS limit";
