@@ -26,20 +26,29 @@ namespace mlstm {
 
 constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in LDS
 
-template <int RT, int WT, bool HILO>
-__global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanArgs a) {
+// A chunk is staged in 128 / PS pieces of PS positions (the contraction over positions is a plain sum): the
+// smaller the piece, the smaller the LDS tiles and the prefetch registers, but the more barriers per chunk.
+// Measured on MI355X (B=4, S=16384, NH=8, 256/512): the backward scan (78 KB of LDS with whole chunks) gains 16 %
+// from a register cap that lets two workgroups share a CU, one's matrix work overlapping the other's staging and
+// memory waits; the forward scan (115 KB with the bf16 remainder tile) would need half-chunk pieces for that and
+// loses more to the extra barriers than it gains, so it keeps whole chunks and one workgroup per CU.
+template <int RT, int WT, bool HILO, int PS>
+__global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
+    __attribute__((amdgpu_waves_per_eu(HILO ? 1 : 2, HILO ? 1 : 2))) void scan_kernel(ScanArgs a) {
   constexpr int WC = WT / 64;
   constexpr int NT = 64 * (RT / 64) * WC;
   constexpr int XS = RT + 16;  // LDS row strides (elements); +16 keeps 4 consecutive rows on distinct banks
   constexpr int YS = WT + 16;
-  constexpr int XV = 128 * RT / 8 / NT;  // 16-byte vectors per thread per chunk
-  constexpr int YV = 128 * WT / 8 / NT;
+  constexpr int XV = PS * RT / 8 / NT;   // 16-byte vectors per thread per piece
+  constexpr int YV = PS * WT / 8 / NT;
+  constexpr int NP = kChunk / PS;        // pieces per chunk
   constexpr int XROWS = NT / (RT / 8);   // rows covered by one sweep of the workgroup over X
+  static_assert(XV >= 1 && YV >= 1 && PS % 16 == 0, "piece too small for this tile");
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint16_t* Xs = (uint16_t*)smem_raw;
-  uint16_t* Yh = Xs + 128 * XS;
-  uint16_t* Yl = Yh + 128 * YS;
-  float* npart = (float*)(Yl + (HILO ? 128 * YS : 0));  // [XROWS][RT] partial sums of the n update
+  uint16_t* Yh = Xs + PS * XS;
+  uint16_t* Yl = Yh + PS * YS;
+  float* npart = (float*)(Yl + (HILO ? PS * YS : 0));  // [XROWS][RT] partial sums of the n update
   float* gl = npart + XROWS * RT;                       // [kGBlock] decay factors of the next chunks, in scan order
 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
@@ -91,12 +100,12 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   float xsc[XV], ysc[YV], ynr[YV];
   // The prefetch only LOADS (raw scale factors included): any arithmetic on a loaded value here would make the
   // wave wait for the whole batch of loads before it starts the matrix work they are meant to overlap with.
-  auto prefetch = [&](int c) {
+  auto prefetch = [&](int c, int piece) {
 #pragma unroll
     for (int v = 0; v < XV; ++v) {
       const int idx = tid + v * NT;
       const int j = idx / (RT / 8), cv = idx % (RT / 8);
-      const int t = c * kChunk + j;
+      const int t = c * kChunk + piece * PS + j;
       xr[v] = t < S ? *(const uint4*)(Xg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
       if (do_n) xsc[v] = t < S ? a.scale_a[bh * Sp + t] : 0.f;
     }
@@ -104,7 +113,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
     for (int v = 0; v < YV; ++v) {
       const int idx = tid + v * NT;
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
-      const int t = c * kChunk + j;
+      const int t = c * kChunk + piece * PS + j;
       yr[v] = t < S ? *(const uint4*)(Yg + (size_t)t * DHHV + cv * 8) : make_uint4(0, 0, 0, 0);
       ysc[v] = t < S ? a.scale_a[bh * Sp + t] : 0.f;
       if (a.backward && a.nrow != nullptr) ynr[v] = a.nrow[bh * Sp + t];
@@ -112,13 +121,14 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
   };
 
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
-  prefetch(c_first);
-  for (int it = 0; it < NC; ++it) {
+  prefetch(c_first, 0);
+  for (int hit = 0; hit < NC * NP; ++hit) {
+    const int it = hit / NP, piece = hit % NP;
     const int c = c_first + it * c_step;
     // The decay factors come from LDS, a block of chunks at a time: read straight from global memory inside the
     // loop, the factor would sit behind the prefetch of the next chunk (loads complete in order) and the matrix
     // work would wait for the whole prefetch in every iteration.
-    if ((it & (kGBlock - 1)) == 0) {
+    if (piece == 0 && (it & (kGBlock - 1)) == 0) {
       __syncthreads();
       for (int k = tid; k < kGBlock && it + k < NC; k += NT) gl[k] = a.gbar[(size_t)bh * NC + c + k * c_step];
       // visible after the barrier that follows the staging below
@@ -167,10 +177,10 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
       if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     }
     __syncthreads();
-    if (it + 1 < NC) prefetch(c + c_step);
+    if (hit + 1 < NC * NP) prefetch(piece + 1 < NP ? c : c + c_step, piece + 1 < NP ? piece + 1 : 0);
 
     // ---- emit the state before this chunk's update as bf16 operand fragments
-    {
+    if (piece == 0) {
       const size_t ND = DHQK / 16, NW = DHHV / 32;
       uint4* st = (uint4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
 #pragma unroll
@@ -189,17 +199,19 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
           }
         }
     }
-    // ---- decay, then accumulate X^T (scale . Y) over the 128 positions of the chunk
-    const float g = gl[it & (kGBlock - 1)];
+    // ---- decay (once per chunk), then accumulate X^T (scale . Y) over the positions of this piece
+    const float g = piece == 0 ? gl[it & (kGBlock - 1)] : 1.f;
+    if (piece == 0) {
 #pragma unroll
-    for (int db = 0; db < 2; ++db)
+      for (int db = 0; db < 2; ++db)
 #pragma unroll
-      for (int wb = 0; wb < 2; ++wb) acc[db][wb] *= g;
+        for (int wb = 0; wb < 2; ++wb) acc[db][wb] *= g;
+    }
 
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
 #pragma unroll
-    for (int js = 0; js < 8; ++js) {
+    for (int js = 0; js < PS / 16; ++js) {
       Frag A[2], Bh[2], Bl[2];
 #pragma unroll
       for (int db = 0; db < 2; ++db) {
@@ -227,7 +239,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64)) void scan_kernel(ScanAr
     }
     // ---- normaliser vector (forward, first column tile only): n = gbar n + sum_j abar_j k_j
     if (do_n && tid < RT) {
-      a.nstates[((size_t)bh * NC + c) * DHQK + d_tile + tid] = nval;
+      if (piece == 0) a.nstates[((size_t)bh * NC + c) * DHQK + d_tile + tid] = nval;
       float s = 0.f;
 #pragma unroll
       for (int g2 = 0; g2 < XROWS; ++g2) s += npart[g2 * RT + tid];
@@ -255,13 +267,14 @@ template <int RT, int WT, bool HILO>
 static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
   constexpr int NT = 64 * (RT / 64) * (WT / 64);
   constexpr int XROWS = NT / (RT / 8);
-  const size_t smem = (size_t)128 * (RT + 16) * 2 + (size_t)128 * (WT + 16) * 2 * (HILO ? 2 : 1) +
+  constexpr int PS = 128;
+  const size_t smem = (size_t)PS * (RT + 16) * 2 + (size_t)PS * (WT + 16) * 2 * (HILO ? 2 : 1) +
                       (size_t)(XROWS * RT + kGBlock) * 4;
-  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "scan: cannot raise the dynamic LDS limit";
   dim3 grid(a.DHQK / RT, a.DHHV / WT, BH);
-  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO>), grid, dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO, PS>), grid, dim3(NT), smem, stream, a);
   return nullptr;
 }
 
