@@ -164,15 +164,19 @@ def mlstm_chunkwise__hip_xl_chunk(
     eps: float = 1e-6,
     chunk_size: int = 128,
     autocast_kernel_dtype: torch.dtype = torch.float32,
+    any_sequence_length: bool = False,
     **tuning_kwargs,
 ):
     """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
     ``(H, (C_last fp32 (B,NH,DHQK,DHHV), n_last fp32 (B,NH,DHQK), m_last fp32 (B,NH,1)))``.
-    The matrix kernels multiply in bf16 with fp32 accumulation whatever the input dtype."""
+    The matrix kernels multiply in bf16 with fp32 accumulation whatever the input dtype.
+    ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
+    tail themselves, so every S >= 1 is one call."""
     for key in tuning_kwargs:
         if key not in _IGNORED_TUNING_KWARGS:
             raise TypeError(f"mlstm_chunkwise__hip_xl_chunk() got an unexpected keyword argument '{key}'")
-    validate_xl_chunk_shapes(q.shape[2], chunk_size)
+    if not any_sequence_length:
+        validate_xl_chunk_shapes(q.shape[2], chunk_size)
     fn = _get_fwbw(autocast_kernel_dtype, False, True)
     H, c_last, n_last, m_last = fn.apply(q, k, v, i, f, c_initial, n_initial, m_initial, return_last_states, eps)
     if return_last_states:
@@ -194,15 +198,23 @@ def mlstm_siging_chunkwise__hip_xl_chunk(
     normalize: bool = True,
     chunk_size: int = 128,
     autocast_kernel_dtype: torch.dtype = torch.float32,
+    any_sequence_length: bool = False,
     **tuning_kwargs,
 ):
-    """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``."""
+    """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``.
+    ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules, as for the exp gate."""
     for key in tuning_kwargs:
         if key not in _IGNORED_TUNING_KWARGS:
             raise TypeError(f"mlstm_siging_chunkwise__hip_xl_chunk() got an unexpected keyword argument '{key}'")
-    validate_xl_chunk_shapes(q.shape[2], chunk_size)
+    if not any_sequence_length:
+        validate_xl_chunk_shapes(q.shape[2], chunk_size)
     fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize))
     H, c_last, n_last, _ = fn.apply(q, k, v, i, f, c_initial, n_initial, None, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last)
     return H
+
+
+# the kernels mask a ragged last chunk themselves: sequence-length adapters may hand over any S >= 1 in one call
+mlstm_chunkwise__hip_xl_chunk.supports_any_sequence_length = True
+mlstm_siging_chunkwise__hip_xl_chunk.supports_any_sequence_length = True

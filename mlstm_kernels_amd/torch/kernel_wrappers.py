@@ -28,7 +28,11 @@ def wrap_chunkwise__arbitrary_sequence_length(
 ):
     """Process a sequence of any length S >= 1: the chunkwise kernel consumes the longest prefix that is a
     multiple of chunk_size, then of chunk_size/2, ... down to 16; the last < 16 tokens go through the token
-    loop; S == 1 goes straight to the step kernel.  States are threaded through all parts."""
+    loop; S == 1 goes straight to the step kernel.  States are threaded through all parts.
+
+    A chunkwise kernel that masks a ragged tail itself announces it with the function attribute
+    ``supports_any_sequence_length``; it then gets the whole sequence in ONE call (keyword
+    ``any_sequence_length=True``) instead of the chunk-halving loop plus the per-token loop."""
     B, NH, S, DHQK = k.shape
     DHHV = v.shape[-1]
     dev = k.device
@@ -41,6 +45,13 @@ def wrap_chunkwise__arbitrary_sequence_length(
             q=q.squeeze(2), k=k.squeeze(2), v=v.squeeze(2), i=i, f=f, c=c_state, n=n_state, m=m_state, eps=eps
         )
         h_out = h_out[:, :, None, :]
+    elif getattr(mlstm_chunkwise_kernel, "supports_any_sequence_length", False):
+        h_out, (c_state, n_state, m_state) = mlstm_chunkwise_kernel(
+            q=q.contiguous(), k=k.contiguous(), v=v.contiguous(), f=f.contiguous(), i=i.contiguous(),
+            c_initial=c_state, n_initial=n_state, m_initial=m_state,
+            chunk_size=chunk_size, return_last_states=True, autocast_kernel_dtype=autocast_kernel_dtype, eps=eps,
+            any_sequence_length=True,
+        )
     else:
         assert S > 1, f"Received empty sequence (S={S}), require at least single element in the sequence."
         pieces = []

@@ -140,6 +140,31 @@ def test_arbitrary_sequence_length_wrapper(S):
     torch.testing.assert_close(m, m_r, rtol=1e-9, atol=1e-9)
 
 
+def test_arbitrary_sequence_length_wrapper_hands_whole_sequence_to_a_capable_kernel():
+    """A chunkwise kernel that announces `supports_any_sequence_length` gets ONE call with the whole sequence."""
+    calls = []
+
+    def kernel(**kw):
+        calls.append(kw)
+        return O.mlstm_chunkwise__native_custbw(**{k_: v_ for k_, v_ in kw.items() if k_ != "any_sequence_length"}, )
+
+    kernel.supports_any_sequence_length = True
+    S = 96   # a length the oracle's chunkwise formulation accepts in one piece (chunk 32), so the fake can delegate
+    q, k, v, i, f = make_qkvif(1, 2, S, 32, 32, seed=5, dtype=torch.float64)
+    i, f = i.double(), f.double()
+
+    def fail(**kw):
+        raise AssertionError("token loop must not run")
+
+    H, (C, n, m) = wrap_chunkwise__arbitrary_sequence_length(
+        mlstm_chunkwise_kernel=kernel, mlstm_sequence_kernel=fail, mlstm_step_kernel=fail,
+        q=q, k=k, v=v, f=f, i=i, chunk_size=32, dtype_state=torch.float64)
+    assert len(calls) == 1 and calls[0]["any_sequence_length"] is True and calls[0]["q"].shape[2] == S
+    H_ref, (C_r, n_r, m_r) = O.recurrent_sequence(q, k, v, i, f)
+    torch.testing.assert_close(H, H_ref, rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(C, C_r, rtol=1e-9, atol=1e-9)
+
+
 def test_backend_inference_mode_threads_states():
     q, k, v, i, f = make_qkvif(1, 2, 100, 32, 32, seed=3, dtype=torch.float32)
     backend = mLSTMBackend(mLSTMBackendConfig(chunkwise_kernel="chunkwise--native_custbw", sequence_kernel="native_sequence__native",
