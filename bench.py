@@ -152,40 +152,68 @@ def main():
     del q, k, v, i, f, dH
     torch.cuda.empty_cache()
 
-    # ---- decode step: chunkwise prefill, then consecutive in-place steps
-    Bd = DECODE_B
-    qp, kp, vp = rn(Bd, NH, DECODE_PREFILL, DHQK).bfloat16(), rn(Bd, NH, DECODE_PREFILL, DHQK).bfloat16(), rn(Bd, NH, DECODE_PREFILL, DHHV).bfloat16()
-    ip, fp = rn(Bd, NH, DECODE_PREFILL), 3 + rn(Bd, NH, DECODE_PREFILL)
-    with torch.no_grad():
-        _, (c, n, m) = mlstm_chunkwise__hip_xl_chunk(qp, kp, vp, ip, fp, return_last_states=True, chunk_size=CHUNK)
-    del qp, kp, vp, ip, fp
-    total = DECODE_WARMUP + DECODE_STEPS
-    qs, ks, vs = rn(total, Bd, NH, DHQK).bfloat16(), rn(total, Bd, NH, DHQK).bfloat16(), rn(total, Bd, NH, DHHV).bfloat16()
-    is_, fs = rn(total, Bd, NH, 1), 3 + rn(total, Bd, NH, 1)
-    n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
-    _lib.profile_read()
-    t_dec = 0.0
-    for t in range(total):
-        if t == DECODE_WARMUP:
+    # ---- decode step: chunkwise prefill, then consecutive in-place steps (state carried, n/m ping-pong)
+    def bench_decode(Bd, graph):
+        qp, kp, vp = rn(Bd, NH, DECODE_PREFILL, DHQK).bfloat16(), rn(Bd, NH, DECODE_PREFILL, DHQK).bfloat16(), rn(Bd, NH, DECODE_PREFILL, DHHV).bfloat16()
+        ip, fp = rn(Bd, NH, DECODE_PREFILL), 3 + rn(Bd, NH, DECODE_PREFILL)
+        with torch.no_grad():
+            _, (c, n, m) = mlstm_chunkwise__hip_xl_chunk(qp, kp, vp, ip, fp, return_last_states=True, chunk_size=CHUNK)
+        del qp, kp, vp, ip, fp
+        total = DECODE_WARMUP + DECODE_STEPS
+        qs, ks, vs = rn(total, Bd, NH, DHQK).bfloat16(), rn(total, Bd, NH, DHQK).bfloat16(), rn(total, Bd, NH, DHHV).bfloat16()
+        is_, fs = rn(total, Bd, NH, 1), 3 + rn(total, Bd, NH, 1)
+        n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
+        step_bytes = STEP_BYTES_PER_BH * Bd * NH
+        if graph:
+            # two steps (n/m ping-pong) per graph, tokens in static buffers refreshed by device-side copies
+            sq, sk, sv = qs[:2].clone(), ks[:2].clone(), vs[:2].clone()
+            si, sf = is_[:2].clone(), fs[:2].clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                mlstm_recurrent_step__hip_fw(c, n, m, sq[0], sk[0], sv[0], si[0], sf[0], matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
+                mlstm_recurrent_step__hip_fw(c, n_alt, m_alt, sq[1], sk[1], sv[1], si[1], sf[1], matC_new=c, vecN_new=n, scaM_new=m)
+            torch.cuda.current_stream().wait_stream(side)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                mlstm_recurrent_step__hip_fw(c, n, m, sq[0], sk[0], sv[0], si[0], sf[0], matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
+                mlstm_recurrent_step__hip_fw(c, n_alt, m_alt, sq[1], sk[1], sv[1], si[1], sf[1], matC_new=c, vecN_new=n, scaM_new=m)
+            for t in range(0, total, 2):
+                if t == DECODE_WARMUP:
+                    torch.cuda.synchronize()
+                    t_dec = time.perf_counter()
+                sq.copy_(qs[t:t + 2]); sk.copy_(ks[t:t + 2]); sv.copy_(vs[t:t + 2]); si.copy_(is_[t:t + 2]); sf.copy_(fs[t:t + 2])
+                g.replay()
             torch.cuda.synchronize()
-            _lib.profile_enable(True)
-            t_dec = time.perf_counter()
-        h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(c, n, m, qs[t], ks[t], vs[t], is_[t], fs[t],
-                                                           matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
-        n_alt, m_alt, n, m = n, m, n_new, m_new
-    torch.cuda.synchronize()
-    dec_ms = (time.perf_counter() - t_dec) / DECODE_STEPS * 1e3
-    _lib.profile_enable(False)
-    st_ms, st_cnt = _lib.profile_read().get("step", (0.0, 1))
-    step_kernel_ms = st_ms / max(st_cnt, 1)
-    step_bytes = STEP_BYTES_PER_BH * Bd * NH
-    decode = {
-        "batch": Bd, "steps": DECODE_STEPS, "ms_per_step": round(dec_ms, 4), "kernel_ms": round(step_kernel_ms, 4),
-        "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
-        "roofline": {"bound": "hbm", "kernel": "step", "achieved": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9, 1),
-                     "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
-    }
+            dec_ms = (time.perf_counter() - t_dec) / DECODE_STEPS * 1e3
+            return {"batch": Bd, "mode": "hip graph (2 steps per replay, incl. token copies)", "ms_per_step": round(dec_ms, 4),
+                    "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s"}
+        _lib.profile_read()
+        t_dec = 0.0
+        for t in range(total):
+            if t == DECODE_WARMUP:
+                torch.cuda.synchronize()
+                _lib.profile_enable(True)
+                t_dec = time.perf_counter()
+            h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(c, n, m, qs[t], ks[t], vs[t], is_[t], fs[t],
+                                                               matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
+            n_alt, m_alt, n, m = n, m, n_new, m_new
+        torch.cuda.synchronize()
+        dec_ms = (time.perf_counter() - t_dec) / DECODE_STEPS * 1e3
+        _lib.profile_enable(False)
+        st_ms, st_cnt = _lib.profile_read().get("step", (0.0, 1))
+        step_kernel_ms = st_ms / max(st_cnt, 1)
+        return {
+            "batch": Bd, "mode": "eager", "steps": DECODE_STEPS, "ms_per_step": round(dec_ms, 4), "kernel_ms": round(step_kernel_ms, 4),
+            "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "roofline": {"bound": "hbm", "kernel": "step", "achieved": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9, 1),
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
+        }
+
+    decode = bench_decode(DECODE_B, graph=False)
+    decode["other_batches"] = [bench_decode(b, graph=g_) for b in (64, 16) for g_ in (False, True)]
+    torch.cuda.empty_cache()
 
     out = {
         "metric": "TFLA fwd+bwd TFLOP/s at B*S=65536 (NH8,256/512); decode-step HBM GB/s",

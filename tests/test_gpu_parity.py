@@ -103,6 +103,52 @@ def test_decode_after_prefill():
     assert (d64(m[:Bo]) - m_r).abs().max() <= 1e-3
 
 
+def test_decode_steps_in_hip_graph():
+    """Two consecutive in-place decode steps (n/m ping-pong between two buffers) captured in one HIP graph; the
+    graph is replayed four times with fresh tokens, with eager work and synchronisations in between, and every
+    replay must reproduce the eager steps bit for bit (the step allocates nothing and records no memset)."""
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw as step_fw
+
+    B, NH, DQK, DHV, R = 16, 8, 256, 512, 4
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    toks = [(rn(B, NH, DQK).bfloat16(), rn(B, NH, DQK).bfloat16(), rn(B, NH, DHV).bfloat16(), rn(B, NH, 1), 3 + rn(B, NH, 1))
+            for _ in range(2 * R)]
+    c0, n0, m0 = rn(B, NH, DQK, DHV), rn(B, NH, DQK), rn(B, NH, 1)
+    # eager run
+    c, n, m = c0.clone(), n0.clone(), m0.clone()
+    n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
+    h_eager = []
+    for t in toks:
+        h, (c, n_new, m_new) = step_fw(c, n, m, *t, matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
+        n_alt, m_alt, n, m = n, m, n_new, m_new
+        h_eager.append(h.clone())
+    c_eager, n_eager, m_eager = c.clone(), n.clone(), m.clone()
+    # graph run: static buffers
+    sc, sn_a, sm_a = c0.clone(), n0.clone(), m0.clone()
+    sn_b, sm_b = torch.empty_like(sn_a), torch.empty_like(sm_a)
+    stok = [[x.clone() for x in toks[0]], [x.clone() for x in toks[1]]]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # warm-up outside the capture, then restore the states
+        step_fw(sc, sn_a, sm_a, *stok[0], matC_new=sc, vecN_new=sn_b, scaM_new=sm_b)
+    torch.cuda.current_stream().wait_stream(side)
+    sc.copy_(c0); sn_a.copy_(n0); sm_a.copy_(m0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        h0, _ = step_fw(sc, sn_a, sm_a, *stok[0], matC_new=sc, vecN_new=sn_b, scaM_new=sm_b)
+        h1, _ = step_fw(sc, sn_b, sm_b, *stok[1], matC_new=sc, vecN_new=sn_a, scaM_new=sm_a)
+    for rep in range(R):
+        for slot in range(2):
+            for dst, src in zip(stok[slot], toks[2 * rep + slot]):
+                dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(h0, h_eager[2 * rep]) and torch.equal(h1, h_eager[2 * rep + 1]), f"replay {rep}"
+        _ = (rn(256, 256) @ rn(256, 256)).sum().item()   # unrelated eager work between replays
+    assert torch.equal(sc, c_eager) and torch.equal(sn_a, n_eager) and torch.equal(sm_a, m_eager)
+
+
 # ------------------------------------------------------------------------------------------ chunkwise forward
 @pytest.mark.parametrize("cfg", [
     dict(B=1, NH=4, S=256, DQK=64, DHV=64, L=64, seed=0, dtype=torch.float32),    # BASELINE config 1 shape
