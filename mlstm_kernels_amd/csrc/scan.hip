@@ -32,10 +32,13 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 // from a register cap that lets two workgroups share a CU, one's matrix work overlapping the other's staging and
 // memory waits; the forward scan (115 KB with the bf16 remainder tile) would need half-chunk pieces for that and
 // loses more to the extra barriers than it gains, so it keeps whole chunks and one workgroup per CU.
-template <int RT, int WT, bool HILO, int PS>
-__global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
-    __attribute__((amdgpu_waves_per_eu(HILO ? 1 : 2, HILO ? 1 : 2))) void scan_kernel(ScanArgs a) {
-  constexpr int WC = WT / 64;
+// WCOLS = value columns per wave (64 or 32): with 32 a 128 x 128 tile takes eight waves, two per SIMD, each with
+// half the staging work and half the accumulators.
+template <int RT, int WT, bool HILO, int PS, int WCOLS>
+__global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
+    __attribute__((amdgpu_waves_per_eu((HILO && WCOLS == 64) ? 1 : 2, (HILO && WCOLS == 64) ? 1 : 2))) void scan_kernel(ScanArgs a) {
+  constexpr int WC = WT / WCOLS;
+  constexpr int NBW = WCOLS / 32;  // 32-column accumulator blocks per wave
   constexpr int NT = 64 * (RT / 64) * WC;
   constexpr int XS = RT + 16;  // LDS row strides (elements); +16 keeps 4 consecutive rows on distinct banks
   constexpr int YS = WT + 16;
@@ -69,15 +72,15 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
   }
   const int bh = bz;
   const int d_tile = bx * RT, w_tile = by * WT;
-  const int d_wave = d_tile + wr * 64, w_wave = w_tile + wc * 64;
+  const int d_wave = d_tile + wr * 64, w_wave = w_tile + wc * WCOLS;
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   const size_t Sp = (size_t)NC * kChunk;
 
-  f32x16 acc[2][2];
+  f32x16 acc[2][NBW];
 #pragma unroll
   for (int db = 0; db < 2; ++db)
 #pragma unroll
-    for (int wb = 0; wb < 2; ++wb) {
+    for (int wb = 0; wb < NBW; ++wb) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         float v0 = 0.f;
@@ -186,7 +189,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
 #pragma unroll
       for (int db = 0; db < 2; ++db)
 #pragma unroll
-        for (int wb = 0; wb < 2; ++wb) {
+        for (int wb = 0; wb < NBW; ++wb) {
           const size_t W32 = (w_wave + 32 * wb) / 32, D16 = (d_wave + 32 * db) / 16;
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
@@ -205,14 +208,14 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
 #pragma unroll
       for (int db = 0; db < 2; ++db)
 #pragma unroll
-        for (int wb = 0; wb < 2; ++wb) acc[db][wb] *= g;
+        for (int wb = 0; wb < NBW; ++wb) acc[db][wb] *= g;
     }
 
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
 #pragma unroll
     for (int js = 0; js < PS / 16; ++js) {
-      Frag A[2], Bh[2], Bl[2];
+      Frag A[2], Bh[NBW], Bl[NBW];
 #pragma unroll
       for (int db = 0; db < 2; ++db) {
         const uint16_t* p = Xs + (16 * js + krow) * XS + (wr * 64 + 32 * db + ncol);
@@ -220,8 +223,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
         A[db].d[1] = lds_read_tr16(p + 4 * XS);
       }
 #pragma unroll
-      for (int wb = 0; wb < 2; ++wb) {
-        const int o = (16 * js + krow) * YS + (wc * 64 + 32 * wb + ncol);
+      for (int wb = 0; wb < NBW; ++wb) {
+        const int o = (16 * js + krow) * YS + (wc * WCOLS + 32 * wb + ncol);
         Bh[wb].d[0] = lds_read_tr16(Yh + o);
         Bh[wb].d[1] = lds_read_tr16(Yh + o + 4 * YS);
         if (HILO) {
@@ -232,7 +235,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
 #pragma unroll
       for (int db = 0; db < 2; ++db)
 #pragma unroll
-        for (int wb = 0; wb < 2; ++wb) {
+        for (int wb = 0; wb < NBW; ++wb) {
           mfma32(acc[db][wb], A[db], Bh[wb]);
           if (HILO) mfma32(acc[db][wb], A[db], Bl[wb]);
         }
@@ -252,7 +255,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
 #pragma unroll
     for (int db = 0; db < 2; ++db)
 #pragma unroll
-      for (int wb = 0; wb < 2; ++wb)
+      for (int wb = 0; wb < NBW; ++wb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int d = d_wave + 32 * db + 8 * (i / 4) + 4 * h + (i % 4);
@@ -265,16 +268,20 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / 64))
 
 template <int RT, int WT, bool HILO>
 static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
-  constexpr int NT = 64 * (RT / 64) * (WT / 64);
+#ifndef MLSTM_SCAN_FW_WCOLS
+#define MLSTM_SCAN_FW_WCOLS 32
+#endif
+  constexpr int WCOLS = HILO ? MLSTM_SCAN_FW_WCOLS : 64;
+  constexpr int NT = 64 * (RT / 64) * (WT / WCOLS);
   constexpr int XROWS = NT / (RT / 8);
   constexpr int PS = 128;
   const size_t smem = (size_t)PS * (RT + 16) * 2 + (size_t)PS * (WT + 16) * 2 * (HILO ? 2 : 1) +
                       (size_t)(XROWS * RT + kGBlock) * 4;
-  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS, WCOLS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "scan: cannot raise the dynamic LDS limit";
   dim3 grid(a.DHQK / RT, a.DHHV / WT, BH);
-  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO, PS>), grid, dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO, PS, WCOLS>), grid, dim3(NT), smem, stream, a);
   return nullptr;
 }
 
