@@ -28,15 +28,21 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 
 // A chunk is staged in 128 / PS pieces of PS positions (the contraction over positions is a plain sum): the
 // smaller the piece, the smaller the LDS tiles and the prefetch registers, but the more barriers per chunk.
-// Measured on MI355X (B=4, S=16384, NH=8, 256/512): the backward scan (78 KB of LDS with whole chunks) gains 16 %
-// from a register cap that lets two workgroups share a CU, one's matrix work overlapping the other's staging and
-// memory waits; the forward scan (115 KB with the bf16 remainder tile) would need half-chunk pieces for that and
-// loses more to the extra barriers than it gains, so it keeps whole chunks and one workgroup per CU.
+// Measured on MI355X (B=4, S=16384, NH=8, 256/512), forward / backward scan in ms:
+//   four waves per 128 x 128 tile, one workgroup per CU (one wave per SIMD)      0.63 / 0.54
+//   four waves, register cap for two workgroups per CU (backward: 78 KB LDS)     -    / 0.46
+//   four waves, half-chunk pieces so that the forward fits twice per CU          0.66 / 0.55
+//   eight waves per tile (64 x 32 per wave), one workgroup per CU                0.46 / 0.41   <- used
+//   eight waves, two workgroups per CU (128 registers per lane)                  -    / 0.45
+// What pays is a second instruction stream per SIMD inside the same workgroup: the phases of a chunk (staging,
+// state emission, matrix work) are serial per wave, and two waves per SIMD overlap one's LDS and conversion
+// latencies with the other's matrix instructions.
+#define SCAN_WPE(HILO_, WCOLS_) ((WCOLS_) == 64 && (HILO_) ? 1 : 2)
 // WCOLS = value columns per wave (64 or 32): with 32 a 128 x 128 tile takes eight waves, two per SIMD, each with
 // half the staging work and half the accumulators.
 template <int RT, int WT, bool HILO, int PS, int WCOLS>
 __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
-    __attribute__((amdgpu_waves_per_eu((HILO && WCOLS == 64) ? 1 : 2, (HILO && WCOLS == 64) ? 1 : 2))) void scan_kernel(ScanArgs a) {
+    __attribute__((amdgpu_waves_per_eu(SCAN_WPE(HILO, WCOLS), SCAN_WPE(HILO, WCOLS)))) void scan_kernel(ScanArgs a) {
   constexpr int WC = WT / WCOLS;
   constexpr int NBW = WCOLS / 32;  // 32-column accumulator blocks per wave
   constexpr int NT = 64 * (RT / 64) * WC;
@@ -271,7 +277,7 @@ static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) 
 #ifndef MLSTM_SCAN_FW_WCOLS
 #define MLSTM_SCAN_FW_WCOLS 32
 #endif
-  constexpr int WCOLS = HILO ? MLSTM_SCAN_FW_WCOLS : 64;
+  constexpr int WCOLS = MLSTM_SCAN_FW_WCOLS;
   constexpr int NT = 64 * (RT / 64) * (WT / WCOLS);
   constexpr int XROWS = NT / (RT / 8);
   constexpr int PS = 128;
