@@ -48,6 +48,21 @@ FLOPS_PER_TOKEN_HEAD["fused_dv"] = FLOPS_PER_TOKEN_HEAD["scan_bw"] + FLOPS_PER_T
 FLOPS_FW = 4 * DHQK * DHHV + CHUNK * (DHQK + DHHV)
 FLOPS_BW = 8 * DHQK * DHHV + CHUNK * (3 * DHQK + 2 * DHHV)
 assert sum(FLOPS_PER_TOKEN_HEAD[n] for n in ("fused_fw", "fused_dv", "par_dq", "par_dk")) == FLOPS_FW + FLOPS_BW
+# algorithmic HBM bytes per launch at this workload: every operand once (bf16 q/k 268 MB, v/dH/H 537 MB, bf16 chunk
+# states 1074 MB per tensor)
+_QB, _VB = B * NH * S * DHQK * 2, B * NH * S * DHHV * 2
+_SB = B * NH * (S // CHUNK) * DHQK * DHHV * 2
+ALG_BYTES = {
+    "scan_fw": _QB + _VB + _SB, "par_h": 2 * _QB + 2 * _VB + _SB,
+    "scan_bw": _QB + _VB + _SB, "par_dv": 2 * _QB + 2 * _VB + _SB,
+    "par_dq": 3 * _QB + 2 * _VB + _SB, "par_dk": 3 * _QB + 2 * _VB + _SB,
+}
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload (calibrated against a
+# copy kernel of known size; summary in profiles/tfla_fwbw_B4_S16384__step_B256__pmc_hbm_traffic.md)
+MEASURED_HBM_BYTES = {
+    "scan_fw": 2012e6, "par_h": 2699e6, "scan_bw": 1947e6, "par_dv": 2735e6, "par_dq": 2976e6, "par_dk": 2969e6,
+    "step": 2163e6,
+}
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # decode step: bytes per (batch, head): C and n read+write fp32, m read+write, q,k,v in, h out (bf16), i,f
@@ -71,15 +86,15 @@ def cpu_baseline(torch):
     f = 3 + torch.randn(1, nh_s, S, generator=g)
     O.chunkwise_bw(q[:, :1, :1024], k[:, :1, :1024], v[:, :1, :1024], i[:, :1, :1024], f[:, :1, :1024], dH[:, :1, :1024], chunk_size=CHUNK)
     times = []
-    for _ in range(3):
+    for _ in range(9):
         t0 = time.perf_counter()
         O.chunkwise_bw(q, k, v, i, f, dH, chunk_size=CHUNK)   # runs the forward (all states) and the backward
         times.append(time.perf_counter() - t0)
-    t = sorted(times)[1]
+    t = sorted(times)[len(times) // 2]
     flops = (FLOPS_FW + FLOPS_BW) * nh_s * S
     return {
         "value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": f"fp32 oracle fwd+bwd on all {B * NH} (batch,head) pairs at S={S}: {t:.2f} s per pass, median of 3 after a warm-up",
+        "sample": f"fp32 oracle fwd+bwd on all {B * NH} (batch,head) pairs at S={S}: {t:.2f} s per pass, median of 9 after a warm-up",
     }
 
 
@@ -146,9 +161,17 @@ def main():
     dom = max((n for n in kernels if n in FLOPS_PER_TOKEN_HEAD), key=lambda n: kernels[n]["avg_ms"])
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["alg_tflops"], "peak": PEAK_BF16_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(kernels[dom]["alg_tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": None,
-        "avg_launch_ms": kernels[dom]["avg_ms"],
+        "unit": "TFLOP/s", "frac": round(kernels[dom]["alg_tflops"] / PEAK_BF16_TFLOPS, 4),
+        "traffic": MEASURED_HBM_BYTES.get(dom), "avg_launch_ms": kernels[dom]["avg_ms"],
     }
+    # the same kernel against the HBM roofline (at 65 flop per byte of materialised-state traffic the step is
+    # bandwidth-bound; both fractions are reported)
+    gbs = ALG_BYTES[dom] / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
+    roofline_hbm = {"bound": "hbm", "kernel": dom, "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_HBM_BYTES.get(dom)}
+    for name, entry in kernels.items():
+        if name in ALG_BYTES:
+            entry["alg_gbs"] = round(ALG_BYTES[name] / (entry["avg_ms"] * 1e-3) / 1e9, 1)
     del q, k, v, i, f, dH
     torch.cuda.empty_cache()
 
@@ -208,7 +231,8 @@ def main():
             "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
             "roofline": {"bound": "hbm", "kernel": "step", "achieved": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None},
+                         "frac": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "traffic": MEASURED_HBM_BYTES["step"] if Bd == DECODE_B else None},
         }
 
     decode = bench_decode(DECODE_B, graph=False)
@@ -222,7 +246,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "mLSTMexp TFLA fwd+bwd, B=4 S=16384 NH=8 DHQK=256 DHHV=512 chunk=128 (BASELINE configs[2]); "
                                "decode step B=256 (configs[4])"},
-        "roofline": roofline, "kernels": kernels, "decode_step": decode,
+        "roofline": roofline, "roofline_hbm": roofline_hbm, "kernels": kernels, "decode_step": decode,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
