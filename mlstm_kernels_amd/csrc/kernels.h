@@ -40,6 +40,9 @@ struct ParHvArgs {
   float qk_scale, eps;
   int sig_gate;
   int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant
+#ifdef MLSTM_PAR_TIMING
+  unsigned long long* timing;  // one-off timing builds: per-wave cycle counts of the phases of one chunk's workgroups
+#endif
 };
 
 struct FusedHvArgs {

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   const int QS = DHQK + 8;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  const int n_region = 64 * (QS > HS ? QS : HS);
+  const int n_region = 64 * QS;
   uint16_t* Ns = (uint16_t*)smem_raw;  // resident Xn rows [64][DHQK] in fragment order
   uint16_t* Ps = Ns + n_region;
   uint16_t* Ts = Ps + 64 * PS;
@@ -57,9 +57,15 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
   const BlockId blk = xcd_block_id();  // halves and column tiles of one chunk share operands: same XCD
+#ifdef MLSTM_PAR_TIMING
+  unsigned long long tph[7] = {0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
+#define MLSTM_PTICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
+#else
+#define MLSTM_PTICK(p_)
+#endif
   const int bh = blk.z, c = blk.y;
-  const int nh = blk.x & 1;            // which half of the chunk's positions
-  const int w_tile = (blk.x >> 1) * WT;
+  const int nh = blk.x;                // which half of the chunk's positions
+  const int NWT = DHHV / WT;           // column tiles, handled one after the other by this workgroup
   const size_t Sp = (size_t)NC * kChunk;
   const size_t gofs = bh * Sp + (size_t)c * kChunk;
   const int t_base = c * kChunk;
@@ -68,7 +74,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   const int ob_lo = IS_DV ? 2 * nh : 0, ob_hi = IS_DV ? 4 : 2 * (nh + 1);
   const uint16_t* Xn_g = (IS_DV ? a.K : a.Q) + (size_t)bh * S * DHQK;
   const uint16_t* Xo_g = (IS_DV ? a.Q : a.K) + (size_t)bh * S * DHQK;
-  const uint16_t* Xw_g = (IS_DV ? a.dH : a.V) + (size_t)bh * S * DHHV + w_tile;
+  const uint16_t* Xw_g = (IS_DV ? a.dH : a.V) + (size_t)bh * S * DHHV;
 
   // ---- phase 0: resident rows, gate vectors (and n_prev) into LDS; first score slab into registers
   constexpr int KV = 128 * 8 / NTH;  // 16-byte vectors per thread per score slab (128 rows x 64 columns)
@@ -84,13 +90,43 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
     }
   };
   load_kslab(0);
+  // state fragments of the first contraction steps of the first column tile: requested up front, together with
+  // everything else this workgroup needs first, so that all of it costs ONE trip to memory (they are consumed in
+  // the main phase, after the score phase)
+  const int m_wave = wave * 64;  // first value column of this wave inside a column tile
+  const int ND = DHQK / 16;
+  const uint4* const st_chunk = (const uint4*)a.states + ((size_t)bh * NC + c) * (size_t)(DHHV / 32) * ND * 64 + lane;
+  Frag ring[PD][2];
+#define MLSTM_LOAD_RING(wt_)                                                                               \
+  {                                                                                                        \
+    const uint4* s0_ = st_chunk + ((size_t)((wt_) * WT + m_wave) / 32 * ND) * 64;                          \
+    _Pragma("unroll") for (int p = 0; p < PD; ++p) {                                                       \
+      ring[p][0].u = s0_[(size_t)p * 64];                                                                  \
+      ring[p][1].u = s0_[(size_t)(ND + p) * 64];                                                           \
+    }                                                                                                      \
+  }
+  MLSTM_LOAD_RING(0)
   {
+    // resident rows: all loads of a batch are issued before the first LDS store (a load-store-load-store loop
+    // would pay the memory latency once per iteration)
     const int vec_per_row = DHQK / 8;
-    for (int idx = tid; idx < 64 * vec_per_row; idx += NTH) {
-      const int j = idx / vec_per_row, cv = idx % vec_per_row;
-      const int t = t_base + n0 + j;
-      const uint4 v = t < S ? *(const uint4*)(Xn_g + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
-      store_perm16(Ns + j * QS, cv, v);
+    constexpr int QB = 8;
+    for (int base = 0; base < 64 * vec_per_row; base += QB * NTH) {
+      u32x4 qrow[QB];
+#pragma unroll
+      for (int u = 0; u < QB; ++u) {
+        const int idx = base + tid + u * NTH;
+        const int j = idx / vec_per_row, cv = idx % vec_per_row;
+        const int t = t_base + n0 + j;
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        qrow[u] = (idx < 64 * vec_per_row && t < S) ? *(const u32x4*)(Xn_g + (size_t)t * DHQK + cv * 8) : z;
+      }
+#pragma unroll
+      for (int u = 0; u < QB; ++u) {
+        const int idx = base + tid + u * NTH;
+        const int j = idx / vec_per_row, cv = idx % vec_per_row;
+        if (idx < 64 * vec_per_row) store_perm16(Ns + j * QS, cv, make_uint4(qrow[u][0], qrow[u][1], qrow[u][2], qrow[u][3]));
+      }
     }
     for (int idx = tid; idx < 128; idx += NTH) {
       uu[idx] = a.g.u[gofs + idx];
@@ -103,26 +139,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
       for (int d = tid; d < DHQK; d += NTH) nperm[perm16(d)] = a.nstates[((size_t)bh * NC + c) * DHQK + d];
   }
 
-  // state fragments of the first contraction steps: requested before the score phase so that their HBM latency
-  // is covered by it (they are consumed in the main phase)
-  const int m_wave = wave * 64;  // first value column of this wave inside the tile
-  const int ND = DHQK / 16;
-  const uint4* st0;
-  const uint4* st1;
-  Frag ring[PD][2];
-  {
-    const size_t NW = DHHV / 32;
-    const uint4* st = (const uint4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
-    const size_t W32 = (size_t)(w_tile + m_wave) / 32;
-    st0 = st + (W32 * ND) * 64 + lane;
-    st1 = st + ((W32 + 1) * ND) * 64 + lane;
-#pragma unroll
-    for (int p = 0; p < PD; ++p) {
-      ring[p][0].u = st0[(size_t)p * 64];
-      ring[p][1].u = st1[(size_t)p * 64];
-    }
-  }
-
+  MLSTM_PTICK(0)
   // ---- phase S: score blocks (32 o x 64 n), dealt round-robin to the waves; contraction over DHQK in slabs of 64
   constexpr int OBW = (4 + NWAVE - 1) / NWAVE;  // score blocks per wave (at most)
   f32x16 sacc[OBW][2];
@@ -160,19 +177,20 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
       }
     }
   }
+  MLSTM_PTICK(1)
   // first value slab into registers while the score matrix is gated
   constexpr int VV = 32 * (WT / 8) / NTH;  // 16-byte vectors per thread per value slab (32 rows x WT columns)
   uint4 vreg[VV];
-  auto load_vslab = [&](int ob) {
+  auto load_vslab = [&](int wt, int ob) {
 #pragma unroll
     for (int v = 0; v < VV; ++v) {
       const int idx = tid + v * NTH;
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
       const int t = t_base + 32 * ob + j;
-      vreg[v] = t < S ? *(const uint4*)(Xw_g + (size_t)t * DHHV + cv * 8) : make_uint4(0, 0, 0, 0);
+      vreg[v] = t < S ? *(const uint4*)(Xw_g + (size_t)t * DHHV + wt * WT + cv * 8) : make_uint4(0, 0, 0, 0);
     }
   };
-  load_vslab(ob_lo);
+  load_vslab(0, ob_lo);
   // gate, mask, round, and write P as Ps[n][o]; forward also accumulates fp32 row sums over j
   {
     float rsum[2] = {0.f, 0.f};
@@ -220,6 +238,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   }
   __syncthreads();
 
+  MLSTM_PTICK(2)
   // ---- phase D (forward): denominators; NTH/64 threads share a row
   if (!IS_DV) {
     constexpr int TPR = NTH / 64;  // threads per row: 4, 2 or 1
@@ -251,7 +270,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
         iv = 1.f / (nmax + a.eps);
       }
       inv[t] = iv;
-      if (w_tile == 0) {
+      {
         a.nrow_out[gofs + n0 + t] = nmax;
         const int tg = t_base + n0 + t;
         if (tg < S) {
@@ -262,53 +281,65 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
     }
   }
 
-  // ---- main phase: Out^T = (State^T Xn^T) * colscale + Xw^T P
-  f32x16 acc[2][2];
+  MLSTM_PTICK(3)
+  // ---- main phase, once per column tile: Out^T = (State^T Xn^T) * colscale + Xw^T P.  The resident rows, the gated
+  // score matrix and the denominators above are shared by all column tiles of this (chunk, position half).
+  const int q16 = (lane >> 4) & 1, i16 = lane & 15;
+  const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
+  for (int wt = 0; wt < NWT; ++wt) {
+    f32x16 acc[2][2];
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+      for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
-  {
-    for (int ds0 = 0; ds0 < ND; ds0 += PD) {
+        for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
+    {
+      const uint4* s0 = st_chunk + ((size_t)(wt * WT + m_wave) / 32 * ND) * 64;
+      for (int ds0 = 0; ds0 < ND; ds0 += PD) {
 #pragma unroll
-      for (int p = 0; p < PD; ++p) {
-        const int ds = ds0 + p;
-        Frag A[2], B[2];
-        A[0] = ring[p][0];
-        A[1] = ring[p][1];
-        if (ds + PD < ND) {
-          ring[p][0].u = st0[(size_t)(ds + PD) * 64];
-          ring[p][1].u = st1[(size_t)(ds + PD) * 64];
+        for (int p = 0; p < PD; ++p) {
+          const int ds = ds0 + p;
+          Frag A[2], B[2];
+          A[0] = ring[p][0];
+          A[1] = ring[p][1];
+          if (ds + PD < ND) {
+            ring[p][0].u = s0[(size_t)(ds + PD) * 64];
+            ring[p][1].u = s0[(size_t)(ND + ds + PD) * 64];
+          }
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + 16 * ds + 8 * h);
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
         }
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + 16 * ds + 8 * h);
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
       }
     }
-  }
+    // the next column tile's first state fragments travel while this tile finishes (the last tile re-requests its
+    // own: an unconditional load keeps the ring in registers)
+    MLSTM_LOAD_RING(wt + 1 < NWT ? wt + 1 : wt)
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const float sc = cs[32 * nb + r];
+    for (int nb = 0; nb < 2; ++nb) {
+      const float sc = cs[32 * nb + r];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= sc;
-  }
-  {
-    const int q16 = (lane >> 4) & 1, i16 = lane & 15;
-    const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
+      for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= sc;
+    }
+    MLSTM_PTICK(4)
     for (int ob = ob_lo; ob < ob_hi; ++ob) {
-      __syncthreads();  // previous slab consumed (first pass: P / inv written, score slabs consumed)
+      __syncthreads();  // slab buffer free (first pass: P / inv written, score slabs consumed; later: staging stored)
 #pragma unroll
       for (int v = 0; v < VV; ++v) {
         const int idx = tid + v * NTH;
         *(uint4*)(Ts + (idx / (WT / 8)) * VS + (idx % (WT / 8)) * 8) = vreg[v];
       }
       __syncthreads();
-      if (ob + 1 < ob_hi) load_vslab(ob + 1);
+      {
+        // next slab of this tile, or the first slab of the next tile (the very last one re-requests itself)
+        const bool more = ob + 1 < ob_hi;
+        const int wt_n = more ? wt : (wt + 1 < NWT ? wt + 1 : wt);
+        load_vslab(wt_n, more ? ob + 1 : ob_lo);
+      }
 #pragma unroll
       for (int jl = 0; jl < 2; ++jl) {
         Frag A[2], B[2];
@@ -326,48 +357,51 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
           for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
       }
     }
-  }
-  __syncthreads();  // resident rows no longer needed: their region becomes the output staging tile
+    MLSTM_PTICK(5)
 
-  // ---- epilogue: (normalise,) round, transpose through LDS, coalesced store
-  uint16_t* Hs = Ns;
+    // ---- epilogue: (normalise,) round, transpose through the slab buffer (32 positions at a time), coalesced store
+    uint16_t* Og = a.Out + (size_t)bh * S * DHHV + wt * WT;
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const int nl = 32 * nb + r;
-    const float iv = IS_DV ? 1.f : inv[nl];
+    for (int nb = 0; nb < 2; ++nb) {
+      __syncthreads();  // slab buffer free (last value slab consumed / previous half stored)
+      const float iv = IS_DV ? 1.f : inv[32 * nb + r];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+      for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
-        *(uint2*)(Hs + nl * HS + w0) =
-            make_uint2(pack_bf16x2(acc[mb][nb][4 * g4 + 0] * iv, acc[mb][nb][4 * g4 + 1] * iv),
-                       pack_bf16x2(acc[mb][nb][4 * g4 + 2] * iv, acc[mb][nb][4 * g4 + 3] * iv));
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
+          *(uint2*)(Ts + r * HS + w0) =
+              make_uint2(pack_bf16x2(acc[mb][nb][4 * g4 + 0] * iv, acc[mb][nb][4 * g4 + 1] * iv),
+                         pack_bf16x2(acc[mb][nb][4 * g4 + 2] * iv, acc[mb][nb][4 * g4 + 3] * iv));
+        }
+      __syncthreads();
+      constexpr int vec_per_row = WT / 8;
+      for (int idx = tid; idx < 32 * vec_per_row; idx += NTH) {
+        const int j = idx / vec_per_row, cv = idx % vec_per_row;
+        const int t = t_base + n0 + 32 * nb + j;
+        if (t < S) *(uint4*)(Og + (size_t)t * DHHV + cv * 8) = *(const uint4*)(Ts + j * HS + cv * 8);
       }
-  }
-  __syncthreads();
-  {
-    uint16_t* Og = a.Out + (size_t)bh * S * DHHV + w_tile;
-    constexpr int vec_per_row = WT / 8;
-    for (int idx = tid; idx < 64 * vec_per_row; idx += NTH) {
-      const int j = idx / vec_per_row, cv = idx % vec_per_row;
-      const int t = t_base + n0 + j;
-      if (t < S) *(uint4*)(Og + (size_t)t * DHHV + cv * 8) = *(const uint4*)(Hs + j * HS + cv * 8);
     }
   }
+#undef MLSTM_LOAD_RING
+  MLSTM_PTICK(6)
+#ifdef MLSTM_PAR_TIMING
+  if (blk.y == a.NC / 2 && blk.z == 0 && lane == 0)
+    for (int p = 0; p < 7; ++p) a.timing[(blk.x * 4 + (wave & 3)) * 8 + p] = tph[p];
+#endif
 }
 
 template <int WT, bool IS_DV, int PD>
 static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
-  const int QS = a.DHQK + 8, HS = WT + 8;
-  const size_t n_region = (size_t)64 * (QS > HS ? QS : HS);
+  const int QS = a.DHQK + 8;
+  const size_t n_region = (size_t)64 * QS;
   const size_t t_region = (128 * 72 > 32 * (WT + 16)) ? 128 * 72 : 32 * (WT + 16);
   const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + (WT / 64) * 64 + a.DHQK) * 4;
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
   if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, IS_DV, PD>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_hv: cannot raise the dynamic LDS limit";
-  dim3 grid(2 * (a.DHHV / WT), a.NC, BH);
+  dim3 grid(2, a.NC, BH);
   hipLaunchKernelGGL((par_hv_kernel<WT, IS_DV, PD>), grid, dim3(WT), smem, stream, a);
   return nullptr;
 }
