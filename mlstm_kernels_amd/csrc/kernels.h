@@ -77,6 +77,9 @@ struct ParQkArgs {
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
   int use_nrow;
+#ifdef MLSTM_PAR_TIMING
+  unsigned long long* timing;  // one-off timing builds
+#endif
 };
 
 struct GateGradArgs {

@@ -24,7 +24,7 @@
 namespace mlstm {
 
 template <int MT, bool IS_DQ>
-__global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
+__global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(MT == 256 ? 2 : 1, MT == 256 ? 2 : 1))) void par_qk_kernel(ParQkArgs a) {
   constexpr int NWAVE = MT / 64;    // each wave owns 64 head-dim rows = 2 MFMA row blocks
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;       // P stored as Ps[n][o]
@@ -55,6 +55,13 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
   const BlockId blk = xcd_block_id();
+#ifdef MLSTM_PAR_TIMING
+  unsigned long long tph[7] = {0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
+  const unsigned long long tstart = tlast;
+#define MLSTM_PTICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
+#else
+#define MLSTM_PTICK(p_)
+#endif
   const int bh = blk.z, c = blk.y;
   const int nh = blk.x & 1;
   const int d_tile = (blk.x >> 1) * MT;
@@ -101,10 +108,10 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
     constexpr int CV = NDT * 64 / NTH;      // state-fragment vectors per thread per slab
     constexpr int NV = 64 * 4 / NTH;        // Xn vectors per thread per slab
     constexpr int OV = 128 * 4 / NTH;       // Xo vectors per thread per slab
-    u32x4 creg[CV];
-    uint4 nreg[NV], oreg[OV];
-    // (a macro, not a lambda: with the arrays captured by reference the compiler kept them in scratch memory)
-#define MLSTM_LOAD_SLAB(slab_)                                                                                       \
+    u32x4 cregA[CV], cregB[CV];
+    uint4 nregA[NV], oregA[OV], nregB[NV], oregB[OV];
+    // (macros, not lambdas: with the arrays captured by reference the compiler kept them in scratch memory)
+#define MLSTM_LOAD_SLAB(slab_, creg, nreg, oreg)                                                                     \
   {                                                                                                                  \
     _Pragma("unroll") for (int v = 0; v < CV; ++v)                                                                   \
         creg[v] = st[((size_t)(slab_) * ND + d_tile / 16) * 64 + tid + v * NTH];                                     \
@@ -121,36 +128,30 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
       oreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHHV + (slab_) * 32 + (idx & 3) * 8) : make_uint4(0, 0, 0, 0); \
     }                                                                                                                \
   }
+    // lanes 32..63 of every state fragment are stored 4 slots off so that the two lane halves a transposing read
+    // touches together fall on different LDS banks
+#define MLSTM_STORE_SLAB(creg, nreg, oreg)                                                                           \
+  {                                                                                                                  \
+    _Pragma("unroll") for (int v = 0; v < CV; ++v) {                                                                 \
+      const int idx = tid + v * NTH;                                                                                 \
+      ((u32x4*)Cf)[idx ^ (((idx >> 5) & 1) << 2)] = creg[v];                                                         \
+    }                                                                                                                \
+    _Pragma("unroll") for (int v = 0; v < NV; ++v) {                                                                 \
+      const int idx = tid + v * NTH;                                                                                 \
+      *(uint4*)(Xn + (idx >> 2) * XS + (idx & 3) * 8) = nreg[v];                                                     \
+    }                                                                                                                \
+    _Pragma("unroll") for (int v = 0; v < OV; ++v) {                                                                 \
+      const int idx = tid + v * NTH;                                                                                 \
+      *(uint4*)(Xo + (idx >> 2) * XS + (idx & 3) * 8) = oreg[v];                                                     \
+    }                                                                                                                \
+  }
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     // transposing read of the staged fragments: lane i16 of a 16-lane block addresses value column
     // k0 + i16/4 and the 4 consecutive head-dim rows n0 + 4*(i16%4) .. +3
     const int d_grp = i16 & 3;
     const int h_src = d_grp & 1, a_src = d_grp >> 1;
-    const int nslab = DHHV / 32;
-    MLSTM_LOAD_SLAB(0)
-    for (int slab = 0; slab < nslab; ++slab) {
-      __syncthreads();
-#pragma unroll
-      for (int v = 0; v < CV; ++v) {
-        // lanes 32..63 of every fragment are stored 4 slots off so that the two lane halves a transposing read
-        // touches together fall on different LDS banks
-        const int idx = tid + v * NTH;
-        ((u32x4*)Cf)[idx ^ (((idx >> 5) & 1) << 2)] = creg[v];
-      }
-#pragma unroll
-      for (int v = 0; v < NV; ++v) {
-        const int idx = tid + v * NTH;
-        *(uint4*)(Xn + (idx >> 2) * XS + (idx & 3) * 8) = nreg[v];
-      }
-#pragma unroll
-      for (int v = 0; v < OV; ++v) {
-        const int idx = tid + v * NTH;
-        *(uint4*)(Xo + (idx >> 2) * XS + (idx & 3) * 8) = oreg[v];
-      }
-      __syncthreads();
-      // unconditional (the last iteration re-fetches its own slab): a conditional prefetch makes the compiler
-      // keep the prefetch registers in scratch memory across the loop back-edge
-      MLSTM_LOAD_SLAB(slab + 1 < nslab ? slab + 1 : slab)
+    const int nslab = DHHV / 32;  // even: DHHV is a multiple of 64
+    auto multiply_slab = [&]() {
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         Frag B[2];
@@ -190,9 +191,29 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
           for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
         }
       }
+    };
+    // two slabs are in flight in registers while a third is multiplied: one memory round trip spans two slab
+    // periods.  The prefetches are unconditional (the last iterations re-fetch the last slab): a conditional
+    // prefetch makes the compiler keep the prefetch registers in scratch memory across the loop back-edge.
+    MLSTM_LOAD_SLAB(0, cregA, nregA, oregA)
+    MLSTM_LOAD_SLAB(1, cregB, nregB, oregB)
+    MLSTM_PTICK(0)
+    for (int slab = 0; slab < nslab; slab += 2) {
+      __syncthreads();
+      MLSTM_STORE_SLAB(cregA, nregA, oregA)
+      __syncthreads();
+      MLSTM_LOAD_SLAB(slab + 2 < nslab ? slab + 2 : nslab - 1, cregA, nregA, oregA)
+      multiply_slab();
+      __syncthreads();
+      MLSTM_STORE_SLAB(cregB, nregB, oregB)
+      __syncthreads();
+      MLSTM_LOAD_SLAB(slab + 3 < nslab ? slab + 3 : nslab - 1, cregB, nregB, oregB)
+      multiply_slab();
     }
   }
+#undef MLSTM_STORE_SLAB
 #undef MLSTM_LOAD_SLAB
+  MLSTM_PTICK(1)
   // column scale of the inter-chunk part
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
@@ -213,6 +234,20 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
     }
   };
   load_zslab(ob_lo);
+  // the x rows of the row dots (q for dQ, k for dK) are fetched now and parked in registers: their memory round
+  // trip overlaps the gating and pass 2 instead of standing alone in the epilogue
+  constexpr int XV = 64 * (MT / 8) / NTH;
+  uint4 xreg[XV];
+  {
+    const uint16_t* Rg = (IS_DQ ? a.Q : a.K) + (size_t)bh * S * DHQK + d_tile;
+#pragma unroll
+    for (int v = 0; v < XV; ++v) {
+      const int idx = tid + v * NTH;
+      const int j = idx / (MT / 8), cv = idx % (MT / 8);
+      const int t = t_base + n0 + j;
+      xreg[v] = t < S ? *(const uint4*)(Rg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
+    }
+  }
   // gate the score matrix: P[o][n] = sacc * exp(u_t - w_j)/sqrt(DHQK) * rho_t for j <= t; store as Ps[n][o]
 #pragma unroll
   for (int k = 0; k < OBW; ++k) {
@@ -248,6 +283,7 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
     }
   }
 
+  MLSTM_PTICK(2)
   // ---- pass 2 over the live chunk positions o: Out^T += Z^T P
   {
     uint16_t* Zs = Cf;
@@ -282,18 +318,15 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
   }
   __syncthreads();
 
+  MLSTM_PTICK(3)
   // ---- epilogue part 1: row dots  sum_d x[n][d] * Out[n][d]  from the fp32 accumulators (x = q for dQ, k for dK).
   // They feed a suffix sum over the whole sequence (dF), where the rounding noise of bf16 outputs would add up
   // like a random walk; the matching x rows are staged in LDS so every lane can read its own row.
   uint16_t* Os = Cf;
-  {
-    const uint16_t* Rg = (IS_DQ ? a.Q : a.K) + (size_t)bh * S * DHQK + d_tile;
-    constexpr int vec_per_row = MT / 8;
-    for (int idx = tid; idx < 64 * vec_per_row; idx += NTH) {
-      const int j = idx / vec_per_row, cv = idx % vec_per_row;
-      const int t = t_base + n0 + j;
-      *(uint4*)(Os + j * OS + cv * 8) = t < S ? *(const uint4*)(Rg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
-    }
+#pragma unroll
+  for (int v = 0; v < XV; ++v) {
+    const int idx = tid + v * NTH;
+    *(uint4*)(Os + (idx / (MT / 8)) * OS + (idx % (MT / 8)) * 8) = xreg[v];
   }
   __syncthreads();
 #pragma unroll
@@ -323,6 +356,7 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
     else atomicAdd(a.rowdot + gofs + n0 + tid, dot);
   }
 
+  MLSTM_PTICK(4)
   // ---- epilogue part 2: round, transpose through LDS, coalesced store
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
@@ -346,6 +380,16 @@ __global__ __launch_bounds__(MT) void par_qk_kernel(ParQkArgs a) {
       if (t < S) *(uint4*)(Og + (size_t)t * DHQK + cv * 8) = *(const uint4*)(Os + j * OS + cv * 8);
     }
   }
+  MLSTM_PTICK(5)
+#ifdef MLSTM_PAR_TIMING
+  if (blk.y == a.NC / 2 && blk.z == 0 && lane == 0)
+    for (int p = 0; p < 6; ++p) a.timing[(blk.x * 4 + (wave & 3)) * 8 + p] = tph[p];
+  if (tid == 0) {
+    const size_t wg = ((size_t)blk.z * a.NC + blk.y) * gridDim.x + blk.x;
+    a.timing[64 + wg * 2] = tstart;
+    a.timing[64 + wg * 2 + 1] = __builtin_amdgcn_s_memtime();
+  }
+#endif
 }
 
 template <int MT, bool IS_DQ>
