@@ -29,10 +29,18 @@
 
 namespace mlstm {
 
+#ifndef MLSTM_PAR_HV_MW256
+#define MLSTM_PAR_HV_MW256 32
+#endif
+
 // PD = how many contraction steps ahead the state fragments are fetched (must divide DHQK / 16).
-template <int WT, bool IS_DV, int PD>
-__global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
-  constexpr int NWAVE = WT / 64;   // each wave owns 64 value columns = 2 MFMA row blocks
+// MW = value columns per wave (64 or 32): WT / MW waves share the tile.
+#define PAR_HV_WPE(WT_, MW_) ((WT_) / (MW_) >= 8 ? 4 : ((WT_) >= 128 ? 2 : 1))
+template <int WT, bool IS_DV, int PD, int MW>
+__global__ __launch_bounds__(64 * (WT / MW))
+    __attribute__((amdgpu_waves_per_eu(PAR_HV_WPE(WT, MW), PAR_HV_WPE(WT, MW)))) void par_hv_kernel(ParHvArgs a) {
+  constexpr int NWAVE = WT / MW;   // each wave owns MW value columns = MB MFMA row blocks
+  constexpr int MB = MW / 32;
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;      // score matrix row stride: P stored as Ps[n][o]
   constexpr int KS = 64 + 8;       // slab row stride of the streamed score operand
@@ -50,8 +58,8 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   float* ww = uu + 128;                 // [128] w_j of the chunk
   float* cs = ww + 128;                 // [64] column scale of this workgroup's positions
   float* inv = cs + 64;                 // forward: [64] 1/(nmax + eps); dV: [128] rho_t of the chunk
-  float* rows = inv + 128;              // [NWAVE][64] partial row sums of Sbar (forward)
-  float* nperm = rows + NWAVE * 64;     // [DHQK] n_prev in fragment order (forward)
+  float* rows = inv + 128;              // [8][32] partial row sums of Sbar per score unit (forward)
+  float* nperm = rows + 8 * 32;         // [DHQK] n_prev in fragment order (forward)
 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -93,24 +101,22 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   // state fragments of the first contraction steps of the first column tile: requested up front, together with
   // everything else this workgroup needs first, so that all of it costs ONE trip to memory (they are consumed in
   // the main phase, after the score phase)
-  const int m_wave = wave * 64;  // first value column of this wave inside a column tile
+  const int m_wave = wave * MW;  // first value column of this wave inside a column tile
   const int ND = DHQK / 16;
   const uint4* const st_chunk = (const uint4*)a.states + ((size_t)bh * NC + c) * (size_t)(DHHV / 32) * ND * 64 + lane;
-  Frag ring[PD][2];
+  Frag ring[PD][MB];
 #define MLSTM_LOAD_RING(wt_)                                                                               \
   {                                                                                                        \
     const uint4* s0_ = st_chunk + ((size_t)((wt_) * WT + m_wave) / 32 * ND) * 64;                          \
-    _Pragma("unroll") for (int p = 0; p < PD; ++p) {                                                       \
-      ring[p][0].u = s0_[(size_t)p * 64];                                                                  \
-      ring[p][1].u = s0_[(size_t)(ND + p) * 64];                                                           \
-    }                                                                                                      \
+    _Pragma("unroll") for (int p = 0; p < PD; ++p)                                                         \
+      _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) ring[p][mb].u = s0_[(size_t)(mb * ND + p) * 64];   \
   }
   MLSTM_LOAD_RING(0)
   {
     // resident rows: all loads of a batch are issued before the first LDS store (a load-store-load-store loop
     // would pay the memory latency once per iteration)
     const int vec_per_row = DHQK / 8;
-    constexpr int QB = 8;
+    constexpr int QB = NTH >= 512 ? 4 : 8;
     for (int base = 0; base < 64 * vec_per_row; base += QB * NTH) {
       u32x4 qrow[QB];
 #pragma unroll
@@ -140,15 +146,14 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   }
 
   MLSTM_PTICK(0)
-  // ---- phase S: score blocks (32 o x 64 n), dealt round-robin to the waves; contraction over DHQK in slabs of 64
-  constexpr int OBW = (4 + NWAVE - 1) / NWAVE;  // score blocks per wave (at most)
-  f32x16 sacc[OBW][2];
+  // ---- phase S: score units (32 o x 32 n; unit u = block ob_lo + u/2, position block u%2), dealt round-robin to the
+  // waves; contraction over DHQK in slabs of 64
+  constexpr int UW = 8 / NWAVE;  // score units per wave
+  f32x16 sacc[UW];
 #pragma unroll
-  for (int k = 0; k < OBW; ++k)
+  for (int k = 0; k < UW; ++k)
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sacc[k][nb][i] = 0.f;
+    for (int i = 0; i < 16; ++i) sacc[k][i] = 0.f;
   const int nslab = DHQK / 64;
   for (int slab = 0; slab < nslab; ++slab) {
     __syncthreads();  // previous slab fully consumed (and phase-0 writes visible on the first pass)
@@ -160,20 +165,19 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
     __syncthreads();
     if (slab + 1 < nslab) load_kslab(slab + 1);
 #pragma unroll
-    for (int k = 0; k < OBW; ++k) {
+    for (int k = 0; k < UW; ++k) {
       // unconditional on purpose: a wave whose block lies above the diagonal multiplies zero rows (its result is
       // dropped at the gating step); a branch here would make the compiler shuttle the score accumulators between
       // the two register files on every iteration
-      const int ob = ob_lo + wave + k * NWAVE;
+      const int u = wave + k * NWAVE;
+      const int ob = ob_lo + (u >> 1), nb = u & 1;
       const int obc = ob < 4 ? ob : 3;
 #pragma unroll
       for (int ds = 0; ds < 4; ++ds) {
-        Frag A, B[2];
+        Frag A, B;
         A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
+        B.u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
+        mfma32(sacc[k], A, B);
       }
     }
   }
@@ -192,48 +196,41 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   };
   load_vslab(0, ob_lo);
   // gate, mask, round, and write P as Ps[n][o]; forward also accumulates fp32 row sums over j
-  {
-    float rsum[2] = {0.f, 0.f};
 #pragma unroll
-    for (int k = 0; k < OBW; ++k) {
-      const int ob = ob_lo + wave + k * NWAVE;
-      if (ob < ob_hi) {
+  for (int k = 0; k < UW; ++k) {
+    const int u = wave + k * NWAVE;
+    const int ob = ob_lo + (u >> 1), nb = u & 1;
+    float rsum = 0.f;
+    if (ob < ob_hi) {
+      const int nl = 32 * nb + r;    // position inside this workgroup's half
+      const int n = n0 + nl;         // position inside the chunk
+      const float un = IS_DV ? ww[n] : uu[n];  // dV: n is the key position j -> w_j ; forward: n = t -> u_t
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
-          const int nl = 32 * nb + r;    // position inside this workgroup's half
-          const int n = n0 + nl;         // position inside the chunk
-          const float un = IS_DV ? ww[n] : uu[n];  // dV: n is the key position j -> w_j ; forward: n = t -> u_t
-#pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            const int o0 = 32 * ob + 8 * g4 + 4 * h;
-            const float4 xo = *(const float4*)((IS_DV ? uu : ww) + o0);
-            const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
-            float rho[4] = {1.f, 1.f, 1.f, 1.f};
-            if (IS_DV) {
-              const float4 rr = *(const float4*)(inv + o0);
-              rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
-            }
-            float pv[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              // exponent u_t - w_j and causal mask j <= t
-              const float ex = IS_DV ? (xov[e] - un) : (un - xov[e]);
-              const bool keep = IS_DV ? (n <= o0 + e) : (o0 + e <= n);
-              const float val = sacc[k][nb][4 * g4 + e] * a.qk_scale * __expf(ex) * rho[e];
-              pv[e] = keep ? val : 0.f;
-              rsum[nb] += pv[e];
-            }
-            *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
-          }
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int o0 = 32 * ob + 8 * g4 + 4 * h;
+        const float4 xo = *(const float4*)((IS_DV ? uu : ww) + o0);
+        const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
+        float rho[4] = {1.f, 1.f, 1.f, 1.f};
+        if (IS_DV) {
+          const float4 rr = *(const float4*)(inv + o0);
+          rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
         }
+        float pv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // exponent u_t - w_j and causal mask j <= t
+          const float ex = IS_DV ? (xov[e] - un) : (un - xov[e]);
+          const bool keep = IS_DV ? (n <= o0 + e) : (o0 + e <= n);
+          const float val = sacc[k][4 * g4 + e] * a.qk_scale * __expf(ex) * rho[e];
+          pv[e] = keep ? val : 0.f;
+          rsum += pv[e];
+        }
+        *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
       }
     }
     if (!IS_DV) {
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        const float tot = rsum[nb] + __shfl_xor(rsum[nb], 32);
-        if (h == 0) rows[wave * 64 + 32 * nb + r] = tot;
-      }
+      const float tot = rsum + __shfl_xor(rsum, 32);
+      if (h == 0) rows[u * 32 + r] = tot;  // units above the diagonal publish zero
     }
   }
   __syncthreads();
@@ -241,7 +238,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   MLSTM_PTICK(2)
   // ---- phase D (forward): denominators; NTH/64 threads share a row
   if (!IS_DV) {
-    constexpr int TPR = NTH / 64;  // threads per row: 4, 2 or 1
+    constexpr int TPR = NTH / 64;  // threads per row: 8, 4, 2 or 1
     const int t = tid / TPR, part = tid % TPR;
     const int seg = DHQK / TPR;
     const uint16_t* qrow = Ns + t * QS + part * seg;
@@ -263,7 +260,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
       if (a.use_nrow) {
         float den = cs[t] * dot;
 #pragma unroll
-        for (int w = 0; w < NWAVE; ++w) den += rows[w * 64 + t];
+        for (int ob4 = 0; ob4 < 4; ++ob4) den += rows[(2 * ob4 + (t >> 5)) * 32 + (t & 31)];
         const float mc = a.g.mcomb[gofs + n0 + t];
         const float floor_v = a.sig_gate ? 1.f : __expf(-mc);
         nmax = fmaxf(fabsf(den), floor_v);
@@ -287,9 +284,9 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
   const int q16 = (lane >> 4) & 1, i16 = lane & 15;
   const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
   for (int wt = 0; wt < NWT; ++wt) {
-    f32x16 acc[2][2];
+    f32x16 acc[MB][2];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -300,17 +297,17 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
 #pragma unroll
         for (int p = 0; p < PD; ++p) {
           const int ds = ds0 + p;
-          Frag A[2], B[2];
-          A[0] = ring[p][0];
-          A[1] = ring[p][1];
+          Frag A[MB], B[2];
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) A[mb] = ring[p][mb];
           if (ds + PD < ND) {
-            ring[p][0].u = s0[(size_t)(ds + PD) * 64];
-            ring[p][1].u = s0[(size_t)(ND + ds + PD) * 64];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) ring[p][mb].u = s0[(size_t)(mb * ND + ds + PD) * 64];
           }
 #pragma unroll
           for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + 16 * ds + 8 * h);
 #pragma unroll
-          for (int mb = 0; mb < 2; ++mb)
+          for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
         }
@@ -323,7 +320,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
     for (int nb = 0; nb < 2; ++nb) {
       const float sc = cs[32 * nb + r];
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= sc;
+      for (int mb = 0; mb < MB; ++mb) acc[mb][nb] *= sc;
     }
     MLSTM_PTICK(4)
     for (int ob = ob_lo; ob < ob_hi; ++ob) {
@@ -342,9 +339,9 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
       }
 #pragma unroll
       for (int jl = 0; jl < 2; ++jl) {
-        Frag A[2], B[2];
+        Frag A[MB], B[2];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int mb = 0; mb < MB; ++mb) {
           const uint16_t* p = Ts + (16 * jl + krow) * VS + (m_wave + 32 * mb + ncol);
           A[mb].d[0] = lds_read_tr16(p);
           A[mb].d[1] = lds_read_tr16(p + 4 * VS);
@@ -352,7 +349,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + 32 * ob + 16 * jl + 8 * h);
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
           for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
       }
@@ -366,7 +363,7 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
       __syncthreads();  // slab buffer free (last value slab consumed / previous half stored)
       const float iv = IS_DV ? 1.f : inv[32 * nb + r];
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
+      for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
           const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
@@ -391,26 +388,27 @@ __global__ __launch_bounds__(WT) void par_hv_kernel(ParHvArgs a) {
 #endif
 }
 
-template <int WT, bool IS_DV, int PD>
+template <int WT, bool IS_DV, int PD, int MW>
 static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
   const int QS = a.DHQK + 8;
   const size_t n_region = (size_t)64 * QS;
   const size_t t_region = (128 * 72 > 32 * (WT + 16)) ? 128 * 72 : 32 * (WT + 16);
-  const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + (WT / 64) * 64 + a.DHQK) * 4;
+  const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + 8 * 32 + a.DHQK) * 4;
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
-  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, IS_DV, PD>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, IS_DV, PD, MW>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_hv: cannot raise the dynamic LDS limit";
   dim3 grid(2, a.NC, BH);
-  hipLaunchKernelGGL((par_hv_kernel<WT, IS_DV, PD>), grid, dim3(WT), smem, stream, a);
+  hipLaunchKernelGGL((par_hv_kernel<WT, IS_DV, PD, MW>), grid, dim3(64 * (WT / MW)), smem, stream, a);
   return nullptr;
 }
 
 template <int WT, bool IS_DV>
 static const char* launch_par_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
   // eight steps ahead (64 registers of fragments in flight per lane) measured 8 % faster than four at 256/512
-  if (a.DHQK % 128 == 0) return launch_par_hv_pd<WT, IS_DV, 8>(a, BH, stream);
-  return launch_par_hv_pd<WT, IS_DV, 4>(a, BH, stream);
+  constexpr int MW = WT == 256 ? MLSTM_PAR_HV_MW256 : 64;
+  if (a.DHQK % 128 == 0) return launch_par_hv_pd<WT, IS_DV, 8, MW>(a, BH, stream);
+  return launch_par_hv_pd<WT, IS_DV, 4, MW>(a, BH, stream);
 }
 
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
