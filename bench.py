@@ -45,9 +45,11 @@ FLOPS_PER_TOKEN_HEAD = {
 # the fused sequential kernels do the work of a scan plus the chunk-parallel kernel that follows it
 FLOPS_PER_TOKEN_HEAD["fused_fw"] = FLOPS_PER_TOKEN_HEAD["scan_fw"] + FLOPS_PER_TOKEN_HEAD["par_h"]
 FLOPS_PER_TOKEN_HEAD["fused_dv"] = FLOPS_PER_TOKEN_HEAD["scan_bw"] + FLOPS_PER_TOKEN_HEAD["par_dv"]
+# dQ and dK run as one launch
+FLOPS_PER_TOKEN_HEAD["par_dqdk"] = FLOPS_PER_TOKEN_HEAD.pop("par_dq") + FLOPS_PER_TOKEN_HEAD.pop("par_dk")
 FLOPS_FW = 4 * DHQK * DHHV + CHUNK * (DHQK + DHHV)
 FLOPS_BW = 8 * DHQK * DHHV + CHUNK * (3 * DHQK + 2 * DHHV)
-assert sum(FLOPS_PER_TOKEN_HEAD[n] for n in ("fused_fw", "fused_dv", "par_dq", "par_dk")) == FLOPS_FW + FLOPS_BW
+assert sum(FLOPS_PER_TOKEN_HEAD[n] for n in ("fused_fw", "fused_dv", "par_dqdk")) == FLOPS_FW + FLOPS_BW
 # algorithmic HBM bytes per launch at this workload: every operand once (bf16 q/k 268 MB, v/dH/H 537 MB, bf16 chunk
 # states 1074 MB per tensor)
 _QB, _VB = B * NH * S * DHQK * 2, B * NH * S * DHHV * 2
@@ -55,12 +57,12 @@ _SB = B * NH * (S // CHUNK) * DHQK * DHHV * 2
 ALG_BYTES = {
     "scan_fw": _QB + _VB + _SB, "par_h": 2 * _QB + 2 * _VB + _SB,
     "scan_bw": _QB + _VB + _SB, "par_dv": 2 * _QB + 2 * _VB + _SB,
-    "par_dq": 3 * _QB + 2 * _VB + _SB, "par_dk": 3 * _QB + 2 * _VB + _SB,
+    "par_dqdk": 4 * _QB + 2 * _VB + 2 * _SB,   # Q, K, V, dH once for both gradients; C and dC states; dQ, dK out
 }
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload (calibrated against a
 # copy kernel of known size; summary in profiles/tfla_fwbw_B4_S16384__step_B256__pmc_hbm_traffic.md)
 MEASURED_HBM_BYTES = {
-    "scan_fw": 2012e6, "par_h": 2699e6, "scan_bw": 1947e6, "par_dv": 2735e6, "par_dq": 2976e6, "par_dk": 2969e6,
+    "scan_fw": 2012e6, "par_h": 2699e6, "scan_bw": 1947e6, "par_dv": 2735e6,
     "step": 2163e6,
 }
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA

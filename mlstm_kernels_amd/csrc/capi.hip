@@ -347,18 +347,14 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   pq.S = S; pq.NC = NC; pq.DHQK = DHQK; pq.DHHV = DHHV;
   pq.qk_scale = qk_scale; pq.eps = eps;
   pq.use_nrow = use_nrow;
+  // dQ and dK in one launch: the workgroups of a chunk run side by side and share the Q, K, V and dH rows they stream
   pq.states = ws.cstates; pq.Out = (uint16_t*)dQ; pq.rowdot = bws.qdq;
+  pq.states2 = bws.dcstates; pq.Out2 = (uint16_t*)dK; pq.rowdot2 = bws.kdk;
   {
-    ProfileScope ps("par_dq", st);
-    if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/true, st)) return fail(e);
+    ProfileScope ps("par_dqdk", st);
+    if (const char* e = mlstm::launch_par_qk_pair(pq, BH, st)) return fail(e);
   }
-  if (check_launch("par_qk dQ")) return 1;
-  pq.states = bws.dcstates; pq.Out = (uint16_t*)dK; pq.rowdot = bws.kdk;
-  {
-    ProfileScope ps("par_dk", st);
-    if (const char* e = mlstm::launch_par_qk(pq, BH, /*is_dq=*/false, st)) return fail(e);
-  }
-  if (check_launch("par_qk dK")) return 1;
+  if (check_launch("par_qk dQ+dK")) return 1;
 
   mlstm::GateGradArgs ga;
   memset(&ga, 0, sizeof(ga));

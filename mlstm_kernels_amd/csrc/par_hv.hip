@@ -37,8 +37,7 @@ namespace mlstm {
 // MW = value columns per wave (64 or 32): WT / MW waves share the tile.
 #define PAR_HV_WPE(WT_, MW_) ((WT_) / (MW_) >= 8 ? 4 : ((WT_) >= 128 ? 2 : 1))
 template <int WT, bool IS_DV, int PD, int MW>
-__global__ __launch_bounds__(64 * (WT / MW))
-    __attribute__((amdgpu_waves_per_eu(PAR_HV_WPE(WT, MW), PAR_HV_WPE(WT, MW)))) void par_hv_kernel(ParHvArgs a) {
+__device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId blk) {
   constexpr int NWAVE = WT / MW;   // each wave owns MW value columns = MB MFMA row blocks
   constexpr int MB = MW / 32;
   constexpr int NTH = 64 * NWAVE;
@@ -64,7 +63,6 @@ __global__ __launch_bounds__(64 * (WT / MW))
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const BlockId blk = xcd_block_id();  // halves and column tiles of one chunk share operands: same XCD
 #ifdef MLSTM_PAR_TIMING
   unsigned long long tph[7] = {0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
 #define MLSTM_PTICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
@@ -386,6 +384,12 @@ __global__ __launch_bounds__(64 * (WT / MW))
   if (blk.y == a.NC / 2 && blk.z == 0 && lane == 0)
     for (int p = 0; p < 7; ++p) a.timing[(blk.x * 4 + (wave & 3)) * 8 + p] = tph[p];
 #endif
+}
+
+template <int WT, bool IS_DV, int PD, int MW>
+__global__ __launch_bounds__(64 * (WT / MW))
+    __attribute__((amdgpu_waves_per_eu(PAR_HV_WPE(WT, MW), PAR_HV_WPE(WT, MW)))) void par_hv_kernel(ParHvArgs a) {
+  par_hv_body<WT, IS_DV, PD, MW>(a, xcd_block_id());  // both halves of a chunk share operands: same XCD
 }
 
 template <int WT, bool IS_DV, int PD, int MW>

@@ -24,7 +24,7 @@
 namespace mlstm {
 
 template <int MT, bool IS_DQ>
-__global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(MT == 256 ? 2 : 1, MT == 256 ? 2 : 1))) void par_qk_kernel(ParQkArgs a) {
+__device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId blk) {
   constexpr int NWAVE = MT / 64;    // each wave owns 64 head-dim rows = 2 MFMA row blocks
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;       // P stored as Ps[n][o]
@@ -54,7 +54,6 @@ __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(MT == 256 ? 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const BlockId blk = xcd_block_id();
 #ifdef MLSTM_PAR_TIMING
   unsigned long long tph[7] = {0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
   const unsigned long long tstart = tlast;
@@ -352,7 +351,7 @@ __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(MT == 256 ? 
     float dot = 0.f;
 #pragma unroll
     for (int w = 0; w < NWAVE; ++w) dot += red[w * 64 + tid];
-    if (gridDim.x == 2) a.rowdot[gofs + n0 + tid] = dot;
+    if (DHQK == MT) a.rowdot[gofs + n0 + tid] = dot;
     else atomicAdd(a.rowdot + gofs + n0 + tid, dot);
   }
 
@@ -385,11 +384,50 @@ __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(MT == 256 ? 
   if (blk.y == a.NC / 2 && blk.z == 0 && lane == 0)
     for (int p = 0; p < 6; ++p) a.timing[(blk.x * 4 + (wave & 3)) * 8 + p] = tph[p];
   if (tid == 0) {
-    const size_t wg = ((size_t)blk.z * a.NC + blk.y) * gridDim.x + blk.x;
+    const size_t wg = ((size_t)blk.z * a.NC + blk.y) * 2 + blk.x + (IS_DQ ? 0 : 8192);
     a.timing[64 + wg * 2] = tstart;
     a.timing[64 + wg * 2 + 1] = __builtin_amdgcn_s_memtime();
   }
 #endif
+}
+
+#define PAR_QK_WPE(MT_) ((MT_) == 256 ? 2 : 1)
+template <int MT, bool IS_DQ>
+__global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(MT), PAR_QK_WPE(MT)))) void par_qk_kernel(ParQkArgs a) {
+  par_qk_body<MT, IS_DQ>(a, xcd_block_id());
+}
+
+// dQ and dK of every chunk in ONE launch: the workgroups of a chunk (both gradients, both position halves, all
+// head-dimension tiles) are neighbours in launch order and run on the same XCD at about the same time, so the Q, K, V
+// and dH rows they all stream are fetched from HBM once and served to the others from the caches.
+template <int MT>
+__global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(MT), PAR_QK_WPE(MT)))) void par_qk_pair_kernel(ParQkArgs a) {
+  BlockId blk = xcd_block_id();
+  const int per = 2 * (a.DHQK / MT);
+  if (blk.x < per) {
+    par_qk_body<MT, true>(a, blk);
+  } else {
+    blk.x -= per;
+    a.states = a.states2;
+    a.Out = a.Out2;
+    a.rowdot = a.rowdot2;
+    par_qk_body<MT, false>(a, blk);
+  }
+}
+
+template <int MT>
+static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t stream) {
+  constexpr int CF = (MT / 16) * 64 * 8;
+  constexpr int sa = CF + 64 * 40 + 128 * 40, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
+  constexpr int sab = sa > sb ? sa : sb;
+  constexpr int stage = sab > sc ? sab : sc;
+  const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;
+  if (hipFuncSetAttribute((const void*)par_qk_pair_kernel<MT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)smem) != hipSuccess)
+    return "par_qk: cannot raise the dynamic LDS limit";
+  dim3 grid(4 * (a.DHQK / MT), a.NC, BH);
+  hipLaunchKernelGGL((par_qk_pair_kernel<MT>), grid, dim3(MT), smem, stream, a);
+  return nullptr;
 }
 
 template <int MT, bool IS_DQ>
@@ -417,6 +455,14 @@ const char* launch_par_qk(const ParQkArgs& a, int BH, bool is_dq, hipStream_t st
   if (a.DHQK % 256 == 0) return launch_par_qk_t<256, false>(a, BH, stream);
   if (a.DHQK % 128 == 0) return launch_par_qk_t<128, false>(a, BH, stream);
   return launch_par_qk_t<64, false>(a, BH, stream);
+}
+
+const char* launch_par_qk_pair(const ParQkArgs& a, int BH, hipStream_t stream) {
+  if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "par_qk: DHQK and DHHV must be multiples of 64";
+  if (a.states2 == nullptr || a.Out2 == nullptr || a.rowdot2 == nullptr) return "par_qk: the dK operands are missing";
+  if (a.DHQK % 256 == 0) return launch_par_qk_pair_t<256>(a, BH, stream);
+  if (a.DHQK % 128 == 0) return launch_par_qk_pair_t<128>(a, BH, stream);
+  return launch_par_qk_pair_t<64>(a, BH, stream);
 }
 
 }  // namespace mlstm
