@@ -21,9 +21,10 @@
 //     below the causal diagonal are computed,
 //   * Xw^T fragments come from row-major slabs through the transposing LDS read; every slab is fetched from
 //     global memory into registers while the previous one is being multiplied.
-// A workgroup owns WT value columns x 64 positions (half a chunk): the tile is small enough (about 72 KB of
-// LDS, < 128 accumulator registers) for two workgroups per CU, which is what hides the global-load latency
-// of one workgroup behind the matrix work of the other.  Its WT/64 waves split the value columns.
+// A workgroup owns 64 positions (half a chunk).  The resident rows, the gated score matrix and (forward) the
+// denominators are built once; then the workgroup walks the value dimension in tiles of WT columns, its WT/MW waves
+// splitting a tile.  The footprint (about 73 KB of LDS) lets two workgroups share a CU; at WT = 256, MW = 32 that is
+// sixteen waves per CU, four instruction streams per SIMD to overlap memory, LDS and matrix latencies.
 #include "common.h"
 #include "kernels.h"
 

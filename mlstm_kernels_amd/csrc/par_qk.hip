@@ -10,14 +10,14 @@
 // with  n = t, o = j, Xn = dH, Xo = V,  Z = K, State = C_prev    (dQ)
 //       n = j, o = t, Xn = V,  Xo = dH, Z = Q, State = dC_next   (dK)
 // and the score matrix  P[o][n] = gate * (Xo Xn^T)  contracted over the DHHV value columns.  One pass over
-// DHHV in slabs of 64 columns feeds BOTH the inter-chunk product and the score matrix from the same Xn slab.
+// DHHV in slabs of 32 columns feeds BOTH the inter-chunk product and the score matrix from the same Xn slab.
 // The state fragments (stored for a contraction over the head dimension) are copied to LDS unchanged and
 // re-read with the transposing LDS read, which hands out operands for a contraction over value columns.
 // Row sums  sum_d x[n][d] * Out[n][d]  (x = q for dQ, k for dK) are emitted for the gate gradients.
 //
-// A workgroup owns MT head-dim rows x 64 positions (half a chunk); every slab is fetched from global memory
-// into registers while the previous one is being multiplied, and the footprint (80 KB of LDS) lets two
-// workgroups share a CU so that one computes while the other waits for memory.
+// A workgroup owns MT head-dim rows x 64 positions (half a chunk); two slabs are in flight from global memory into
+// registers while a third is being multiplied, and the footprint (54 KB of LDS) lets two workgroups share a CU so
+// that one computes while the other waits for memory.  dQ and dK normally run as ONE launch (par_qk_pair_kernel).
 #include "common.h"
 #include "kernels.h"
 
