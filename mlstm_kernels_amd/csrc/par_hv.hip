@@ -104,13 +104,14 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   const int ND = DHQK / 16;
   const uint4* const st_chunk = (const uint4*)a.states + ((size_t)bh * NC + c) * (size_t)(DHHV / 32) * ND * 64 + lane;
   Frag ring[PD][MB];
-#define MLSTM_LOAD_RING(wt_)                                                                               \
+#define MLSTM_LOAD_RING(wt_, stride_)                                                                      \
   {                                                                                                        \
     const uint4* s0_ = st_chunk + ((size_t)((wt_) * WT + m_wave) / 32 * ND) * 64;                          \
     _Pragma("unroll") for (int p = 0; p < PD; ++p)                                                         \
-      _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) ring[p][mb].u = s0_[(size_t)(mb * ND + p) * 64];   \
+      _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                                                    \
+        ring[p][mb].u = s0_[(size_t)(mb * ND + p) * (stride_)];                                            \
   }
-  MLSTM_LOAD_RING(0)
+  MLSTM_LOAD_RING(0, 64)
   {
     // resident rows: all loads of a batch are issued before the first LDS store (a load-store-load-store loop
     // would pay the memory latency once per iteration)
@@ -312,9 +313,15 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         }
       }
     }
-    // the next column tile's first state fragments travel while this tile finishes (the last tile re-requests its
-    // own: an unconditional load keeps the ring in registers)
-    MLSTM_LOAD_RING(wt + 1 < NWT ? wt + 1 : wt)
+    // the next column tile's first state fragments travel while this tile finishes.  The load is unconditional (a
+    // conditional one makes the compiler spill ring registers); after the last tile every ring slot re-requests one
+    // and the same fragment (stride 0), which costs a cache hit instead of 64 KB of fetches from HBM.
+    {
+      const bool more_tiles = wt + 1 < NWT;
+      const int wt_next = more_tiles ? wt + 1 : wt;
+      const int ring_stride = more_tiles ? 64 : 0;
+      MLSTM_LOAD_RING(wt_next, ring_stride)
+    }
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const float sc = cs[32 * nb + r];
