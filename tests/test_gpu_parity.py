@@ -159,6 +159,7 @@ def test_decode_steps_in_hip_graph():
     dict(B=1, NH=2, S=400, DQK=128, DHV=128, L=16, seed=5, dtype=torch.bfloat16),  # ragged tail (3 * 128 + 16)
     dict(B=1, NH=1, S=32, DQK=256, DHV=64, L=32, seed=6, dtype=torch.bfloat16),    # shorter than one chunk
     dict(B=2, NH=2, S=1024, DQK=256, DHV=192, L=128, seed=7, dtype=torch.bfloat16),  # three value slices
+    dict(B=1, NH=2, S=256, DQK=128, DHV=128, L=64, seed=8, dtype=torch.float16),   # fp16 in, fp16 H out
 ])
 def test_chunkwise_forward_exp(cfg):
     exp_op, *_ = _ops()
