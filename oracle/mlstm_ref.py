@@ -16,6 +16,16 @@ Reference files each part follows (paths relative to the reference checkout):
                             fw_kernel_parallel.py:76-256 and
                             mlstm_kernels/torch/chunkwise/triton_xl_chunk_siging/chunkwise_gates.py:72-100
                             (no native chunkwise sig implementation exists in the reference).
+
+How each part is pinned (tests/test_oracle.py, tests/test_golden.py): the decode step by its closed form and a
+hand-computed vector; the forward by three independent formulations (recurrent, quadratic, chunkwise) agreeing in
+fp64 for both gates, plus chunk-size, state-passing and stabiliser-shift invariance; the backward by fp64 autograd
+through an independently written forward and by sum_d k*dK == sum_d v*dV; and the two conventions that only the
+reference can state -- what the forward stores as n_out / m_out, and what the hand-written backward treats as
+constant -- by outputs of the reference's own mlstm_chunkwise_fw / mlstm_chunkwise_bw on seeded inputs
+(tests/golden/reference_native_chunkwise.npz, written by tests/golden/make_reference_vectors.py).  The sigmoid-gate
+chunkwise variant has no native counterpart in the reference to take vectors from; it is pinned by the first two
+groups of checks only.  No function here is "parity unpinned".
 """
 from __future__ import annotations
 

@@ -43,6 +43,100 @@ def test_chunkwise_fixture_oracle(tag, sig):
         torch.testing.assert_close(t, z[f"{tag}_{name}"], rtol=1e-4, atol=1e-4, msg=lambda s: f"{name}: {s}")
 
 
+def _reference_vectors(case):
+    """Outputs of the reference's own native chunkwise forward/backward (tests/golden/make_reference_vectors.py)."""
+    z = np.load(os.path.join(GOLD, "reference_native_chunkwise.npz"))
+    d = {k[len(case) + 1:]: torch.from_numpy(z[k]) for k in z.files if k.startswith(case + "_")}
+    B, NH, S, DQK, DHV, L, init, dcl = (int(x) for x in d.pop("meta"))
+    return d, L, bool(init), bool(dcl)
+
+
+@pytest.mark.parametrize("case", ["a", "b"])
+def test_oracle_matches_reference_native_vectors(case):
+    """Pins the two conventions only the reference can state: the stored normaliser / stabiliser rows (n_out, m_out)
+    and the hand-written backward (constants of the gradient, span of the dF sum).  fp32-stored vectors: 1e-5."""
+    z, L, init, dcl = _reference_vectors(case)
+    z = {k: v.double() for k, v in z.items()}
+    ini = (z["c0"], z["n0"], z["m0"]) if init else (None, None, None)
+    fw = O.chunkwise_fw(z["q"], z["k"], z["v"], z["i"], z["f"], *ini, chunk_size=L)
+    for name in ("H", "n_out", "m_out", "C_last", "n_last", "m_last"):
+        torch.testing.assert_close(fw[name].reshape(z[name].shape), z[name], rtol=1e-5, atol=1e-5, msg=lambda s: f"{name}: {s}")
+    # the chunk size must not matter (the vectors were made with L, the HIP kernels use 128)
+    fw2 = O.chunkwise_fw(z["q"], z["k"], z["v"], z["i"], z["f"], *ini, chunk_size=2 * L)
+    torch.testing.assert_close(fw2["H"], z["H"], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(fw2["n_out"], z["n_out"], rtol=1e-5, atol=1e-5)
+    bw = O.chunkwise_bw(z["q"], z["k"], z["v"], z["i"], z["f"], z["dH"], *ini, z.get("dC_last"), chunk_size=L)
+    names = ["dQ", "dK", "dV", "dI", "dF"] + (["dC0"] if init else [])
+    for name, t in zip(names, bw):
+        torch.testing.assert_close(t, z[name], rtol=1e-5, atol=2e-5, msg=lambda s: f"{name}: {s}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["a", "b"])
+def test_hip_matches_reference_native_vectors(case):
+    from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk
+
+    z, L, init, dcl = _reference_vectors(case)
+    dev = "cuda"
+    q, k, v = (z[x].bfloat16().to(dev).requires_grad_(True) for x in "qkv")
+    i, f = z["i"].to(dev).requires_grad_(True), z["f"].to(dev).requires_grad_(True)
+    kw = {}
+    if init:
+        c0 = z["c0"].to(dev).requires_grad_(True)
+        kw = dict(c_initial=c0, n_initial=z["n0"].to(dev), m_initial=z["m0"].to(dev))
+    H, (C, n, m) = mlstm_chunkwise__hip_xl_chunk(q, k, v, i, f, return_last_states=True, chunk_size=L, **kw)
+    loss = (H.float() * z["dH"].to(dev)).sum()
+    if dcl:
+        loss = loss + (C * z["dC_last"].to(dev)).sum()
+    loss.backward()
+    # tolerances: outputs / gradients 2e-2 (bf16 operands), states 1e-3, gate gradients 5e-2 of their scale
+    assert allclose_frac(H, z["H"], 2e-2, 2e-2) <= 1e-3 and rel_to_scale(H, z["H"]) <= 1e-2
+    assert_state_close(C, z["C_last"], 1e-3, "C_last")
+    assert_state_close(n, z["n_last"], 1e-3, "n_last")
+    assert (m.cpu() - z["m_last"]).abs().max() <= 1e-3
+    for name, t in (("dQ", q), ("dK", k), ("dV", v)):
+        assert allclose_frac(t.grad, z[name], 2e-2, 2e-2) <= 1e-3, name
+        assert rel_to_scale(t.grad, z[name]) <= 1e-2 and rel_norm(t.grad, z[name]) <= 5e-3, name
+    for name, t in (("dI", i), ("dF", f)):
+        assert rel_to_scale(t.grad, z[name]) <= 5e-2, name
+    if init:
+        assert rel_norm(c0.grad, z["dC0"]) <= 5e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["a", "b"])
+def test_hip_stored_rows_match_reference_native_vectors(case):
+    """The optional n_out / m_out outputs of the C entry point (the rows the reference's forward returns as vecN_out and
+    vecM_out, native/fw.py:208-212) against the reference-made vectors: m_out depends on the gates only (1e-4), n_out
+    carries the bf16 rounding of the scores (2e-2)."""
+    from mlstm_kernels_amd import _lib
+    from mlstm_kernels_amd.torch.utils import current_stream_ptr, ptr
+
+    z, L, init, dcl = _reference_vectors(case)
+    dev = torch.device("cuda")
+    q, k, v = (z[x].bfloat16().to(dev).contiguous() for x in "qkv")
+    i, f = z["i"].to(dev).contiguous(), z["f"].to(dev).contiguous()
+    B, NH, S, DHQK = q.shape
+    DHHV = v.shape[-1]
+    c0 = n0 = m0 = None
+    if init:
+        c0, n0, m0 = z["c0"].to(dev).contiguous(), z["n0"].to(dev).contiguous(), z["m0"].reshape(B, NH).to(dev).contiguous()
+    lib = _lib.get_lib()
+    ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
+    n_out = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
+    m_out = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
+    rc = lib.mlstm_hip_chunkwise_fw(ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0), ptr(H), ptr(n_out),
+                                    ptr(m_out), None, None, None, ptr(ws), ws_bytes, 0, B, NH, S, DHQK, DHHV, 1e-6,
+                                    _lib.BF16, _lib.F32, _lib.GATE_EXP, 1, current_stream_ptr(dev))
+    _lib.check(rc, "mlstm_hip_chunkwise_fw")
+    torch.cuda.synchronize()
+    assert (m_out.cpu() - z["m_out"]).abs().max() <= 1e-4
+    torch.testing.assert_close(n_out.cpu(), z["n_out"], rtol=2e-2, atol=2e-2)
+    assert allclose_frac(H, z["H"], 2e-2, 2e-2) <= 1e-3
+
+
 @pytest.mark.gpu
 def test_step_kat_hip():
     from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip
