@@ -74,8 +74,8 @@ struct ParQkArgs {
   const float* nrow;
   uint16_t* Out;            // (B,NH,S,DHQK) bf16: dQ or dK
   float* rowdot;            // [BH][Sp]: sum_d q*dQ (dQ) or sum_d k*dK (dK)
-  const uint16_t* states2;  // launch_par_qk_pair only: the dK operands (dC states, dK, sum_d k*dK); the three
-  uint16_t* Out2;           // fields above are then the dQ operands
+  const uint16_t* states2;  // the dK operands (dC states, dK, sum_d k*dK); states, Out and rowdot above are the
+  uint16_t* Out2;           // dQ operands
   float* rowdot2;
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
@@ -102,7 +102,6 @@ const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 bool fused_hv_supported(int DHQK, int DHHV);
 const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream);
-const char* launch_par_qk(const ParQkArgs& a, int BH, bool is_dq, hipStream_t stream);
 const char* launch_par_qk_pair(const ParQkArgs& a, int BH, hipStream_t stream);
 const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream);
 const char* launch_fill_zero(float* p, size_t n, hipStream_t stream);

@@ -392,11 +392,6 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
 }
 
 #define PAR_QK_WPE(MT_) ((MT_) == 256 ? 2 : 1)
-template <int MT, bool IS_DQ>
-__global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(MT), PAR_QK_WPE(MT)))) void par_qk_kernel(ParQkArgs a) {
-  par_qk_body<MT, IS_DQ>(a, xcd_block_id());
-}
-
 // dQ and dK of every chunk in ONE launch: the workgroups of a chunk (both gradients, both position halves, all
 // head-dimension tiles) are neighbours in launch order and run on the same XCD at about the same time, so the Q, K, V
 // and dH rows they all stream are fetched from HBM once and served to the others from the caches.
@@ -428,33 +423,6 @@ static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t 
   dim3 grid(4 * (a.DHQK / MT), a.NC, BH);
   hipLaunchKernelGGL((par_qk_pair_kernel<MT>), grid, dim3(MT), smem, stream, a);
   return nullptr;
-}
-
-template <int MT, bool IS_DQ>
-static const char* launch_par_qk_t(const ParQkArgs& a, int BH, hipStream_t stream) {
-  constexpr int CF = (MT / 16) * 64 * 8;
-  constexpr int sa = CF + 64 * 40 + 128 * 40, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
-  constexpr int sab = sa > sb ? sa : sb;
-  constexpr int stage = sab > sc ? sab : sc;
-  const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;
-  if (hipFuncSetAttribute((const void*)par_qk_kernel<MT, IS_DQ>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (int)smem) != hipSuccess)
-    return "par_qk: cannot raise the dynamic LDS limit";
-  dim3 grid(2 * (a.DHQK / MT), a.NC, BH);
-  hipLaunchKernelGGL((par_qk_kernel<MT, IS_DQ>), grid, dim3(MT), smem, stream, a);
-  return nullptr;
-}
-
-const char* launch_par_qk(const ParQkArgs& a, int BH, bool is_dq, hipStream_t stream) {
-  if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "par_qk: DHQK and DHHV must be multiples of 64";
-  if (is_dq) {
-    if (a.DHQK % 256 == 0) return launch_par_qk_t<256, true>(a, BH, stream);
-    if (a.DHQK % 128 == 0) return launch_par_qk_t<128, true>(a, BH, stream);
-    return launch_par_qk_t<64, true>(a, BH, stream);
-  }
-  if (a.DHQK % 256 == 0) return launch_par_qk_t<256, false>(a, BH, stream);
-  if (a.DHQK % 128 == 0) return launch_par_qk_t<128, false>(a, BH, stream);
-  return launch_par_qk_t<64, false>(a, BH, stream);
 }
 
 const char* launch_par_qk_pair(const ParQkArgs& a, int BH, hipStream_t stream) {
