@@ -16,8 +16,10 @@
 // the sequence end inside the last chunk get logsig(f) = 0 and it = -inf, i.e. they neither decay nor feed
 // the state, so any sequence length is handled.
 //
-// One workgroup per (batch, head): phase 1 does the within-chunk scans wave-parallel, phase 2 scans the
-// (max,+) recurrence of m over chunks with one wave (the recurrence is associative), phase 3 is elementwise.
+// Two launches, each with one workgroup per (batch, head, group of 16 chunks) so that a small batch still fills
+// the chip: the first does the within-chunk scans (one wave per chunk); the second scans the (max,+) recurrence of m
+// over ALL chunks of its head with one wave (the recurrence is associative and only NC scalars long, so every
+// workgroup of a head repeats it rather than waiting for a neighbour) and finishes its own chunks elementwise.
 #include "common.h"
 #include "kernels.h"
 
@@ -47,81 +49,101 @@ __device__ __forceinline__ float wave_rev_incl_scan(float x, Op op) {
   return x;
 }
 
-__global__ __launch_bounds__(kGateThreads) void gates_kernel(
-    const void* __restrict__ ig, const void* __restrict__ fg, const float* __restrict__ m0,
-    GateBufs gb, float* __restrict__ m_last, int S, int NC, int dtype_gates, int sig_gate) {
-  const int bh = blockIdx.x;
+constexpr int kGateChunks = kGateThreads / kWave;  // chunks per workgroup: one wave each
+
+__global__ __launch_bounds__(kGateThreads) void gates_scan_kernel(
+    const void* __restrict__ ig, const void* __restrict__ fg, GateBufs gb, int S, int NC, int dtype_gates,
+    int sig_gate) {
+  const int bh = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = blockIdx.x * kGateChunks + wave;
+  if (c >= NC) return;
   const size_t Sp = (size_t)NC * kChunk;
-  float* u = gb.u + bh * Sp;          // phase 1: b
+  float* u = gb.u + bh * Sp;          // here: b
   float* wv = gb.w + bh * Sp;
-  float* abar = gb.abar + bh * Sp;    // phase 1: a
-  float* bbar = gb.bbar + bh * Sp;
-  float* mcomb = gb.mcomb + bh * Sp;  // phase 1: b + cummax(it - b)
-  float* gbar = gb.gbar + (size_t)bh * NC;  // phase 1: g
-  float* amax = gb.amax + (size_t)bh * NC;
-  float* mst = gb.mstates + (size_t)bh * (NC + 1);
+  float* abar = gb.abar + bh * Sp;    // here: a
+  float* mcomb = gb.mcomb + bh * Sp;  // here: b + cummax(it - b)
   const float NEG_INF = -__builtin_inff();
   auto add = [](float a, float b) { return a + b; };
   auto mx = [](float a, float b) { return fmaxf(a, b); };
 
-  // ---- phase 1: within-chunk scans, one wave per chunk, two positions per lane
-  for (int c = wave; c < NC; c += kGateThreads / kWave) {
-    const int t0 = c * kChunk + 2 * lane;
-    float lf[2], it[2];
+  // within-chunk scans, one wave per chunk, two positions per lane
+  const int t0 = c * kChunk + 2 * lane;
+  float lf[2], it[2];
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const int t = t0 + e;
-      if (t < S) {
-        const size_t o = (size_t)bh * S + t;
-        lf[e] = log_sigmoid(load_scalar(fg, o, dtype_gates));
-        const float iv = load_scalar(ig, o, dtype_gates);
-        it[e] = sig_gate ? log_sigmoid(iv) : iv;
-      } else {
-        lf[e] = 0.f;
-        it[e] = NEG_INF;
-      }
-    }
-    const float pair = lf[0] + lf[1];
-    const float incl = wave_incl_scan(pair, add, 0.f);
-    const float b1 = incl, b0 = (incl - pair) + lf[0];
-    const float g = __shfl(incl, 63);
-    const float rincl = wave_rev_incl_scan(pair, add);
-    const float suf1 = rincl - pair, suf0 = suf1 + lf[1];
-    const float a0 = suf0 + it[0], a1 = suf1 + it[1];
-    const float x0 = it[0] - b0, x1 = it[1] - b1;
-    const float pm = wave_incl_scan(fmaxf(x0, x1), mx, NEG_INF);
-    float pm_excl = __shfl_up(pm, 1);
-    if (lane == 0) pm_excl = NEG_INF;
-    const float cm0 = fmaxf(pm_excl, x0), cm1 = pm;
-    const float am = wave_max(fmaxf(a0, a1));
-    *(float2*)(u + t0) = make_float2(b0, b1);
-    *(float2*)(mcomb + t0) = make_float2(b0 + cm0, b1 + cm1);
-    *(float2*)(abar + t0) = make_float2(a0, a1);
-    *(float2*)(wv + t0) = make_float2(b0 - it[0], b1 - it[1]);
-    if (lane == 0) {
-      gbar[c] = g;
-      amax[c] = am;
+  for (int e = 0; e < 2; ++e) {
+    const int t = t0 + e;
+    if (t < S) {
+      const size_t o = (size_t)bh * S + t;
+      lf[e] = log_sigmoid(load_scalar(fg, o, dtype_gates));
+      const float iv = load_scalar(ig, o, dtype_gates);
+      it[e] = sig_gate ? log_sigmoid(iv) : iv;
+    } else {
+      lf[e] = 0.f;
+      it[e] = NEG_INF;
     }
   }
-  __syncthreads();
+  const float pair = lf[0] + lf[1];
+  const float incl = wave_incl_scan(pair, add, 0.f);
+  const float b1 = incl, b0 = (incl - pair) + lf[0];
+  const float g = __shfl(incl, 63);
+  const float rincl = wave_rev_incl_scan(pair, add);
+  const float suf1 = rincl - pair, suf0 = suf1 + lf[1];
+  const float a0 = suf0 + it[0], a1 = suf1 + it[1];
+  const float x0 = it[0] - b0, x1 = it[1] - b1;
+  const float pm = wave_incl_scan(fmaxf(x0, x1), mx, NEG_INF);
+  float pm_excl = __shfl_up(pm, 1);
+  if (lane == 0) pm_excl = NEG_INF;
+  const float cm0 = fmaxf(pm_excl, x0), cm1 = pm;
+  const float am = wave_max(fmaxf(a0, a1));
+  *(float2*)(u + t0) = make_float2(b0, b1);
+  *(float2*)(mcomb + t0) = make_float2(b0 + cm0, b1 + cm1);
+  *(float2*)(abar + t0) = make_float2(a0, a1);
+  *(float2*)(wv + t0) = make_float2(b0 - it[0], b1 - it[1]);
+  if (lane == 0) {
+    gb.graw[(size_t)bh * NC + c] = g;
+    gb.amax[(size_t)bh * NC + c] = am;
+  }
+}
 
-  // ---- phase 2: m_c = max(g_c + m_{c-1}, amax_c) over chunks; (G, A) pairs compose associatively:
+__global__ __launch_bounds__(kGateThreads) void gates_finish_kernel(const float* __restrict__ m0, GateBufs gb,
+                                                                    float* __restrict__ m_last, int NC, int sig_gate) {
+  __shared__ float msh[kGateChunks + 1];  // m before the chunks of this workgroup, and after its last one
+  const int bh = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c_first = blockIdx.x * kGateChunks;
+  const int c_end = min(c_first + kGateChunks, NC);
+  const size_t Sp = (size_t)NC * kChunk;
+  float* u = gb.u + bh * Sp;
+  float* abar = gb.abar + bh * Sp;
+  float* bbar = gb.bbar + bh * Sp;
+  float* mcomb = gb.mcomb + bh * Sp;
+  const float* graw = gb.graw + (size_t)bh * NC;
+  const float* amax = gb.amax + (size_t)bh * NC;
+  float* gbar = gb.gbar + (size_t)bh * NC;
+  float* mst = gb.mstates + (size_t)bh * (NC + 1);
+  const float NEG_INF = -__builtin_inff();
+
+  // m_c = max(g_c + m_{c-1}, amax_c) over the chunks of the head; (G, A) pairs compose associatively:
   //      (G1, A1) then (G2, A2)  ==  (G1 + G2, max(A1 + G2, A2))
   if (wave == 0) {
-    const float m_init = (m0 != nullptr && !sig_gate) ? m0[bh] : 0.f;
-    const int R = (NC + 63) / 64;
-    const int c_lo = min(lane * R, NC), c_hi = min(c_lo + R, NC);
     if (sig_gate) {
-      for (int c = c_lo; c < c_hi; ++c) {
+      for (int c = c_first + lane; c < c_end; c += kWave) {
         mst[c] = 0.f;
-        gbar[c] = expf(gbar[c]);
+        gbar[c] = expf(graw[c]);
       }
-      if (lane == 63) mst[NC] = 0.f;
+      if (lane < kGateChunks + 1) msh[lane] = 0.f;
+      if (c_end == NC && lane == 0) {
+        mst[NC] = 0.f;
+        if (m_last != nullptr) m_last[bh] = 0.f;
+      }
     } else {
+      const float m_init = m0 != nullptr ? m0[bh] : 0.f;
+      const int R = (NC + 63) / 64;
+      const int c_lo = min(lane * R, NC), c_hi = min(c_lo + R, NC);
       float G = 0.f, A = NEG_INF;
       for (int c = c_lo; c < c_hi; ++c) {
-        const float gc = gbar[c];
+        const float gc = graw[c];
         A = fmaxf(A + gc, amax[c]);
         G += gc;
       }
@@ -140,22 +162,29 @@ __global__ __launch_bounds__(kGateThreads) void gates_kernel(
       }
       float m = fmaxf(m_init + Gex, Aex);
       for (int c = c_lo; c < c_hi; ++c) {
-        const float gc = gbar[c];
+        const float gc = graw[c];
         const float mn = fmaxf(m + gc, amax[c]);
-        mst[c] = m;
-        gbar[c] = expf(gc + m - mn);
+        if (c >= c_first && c < c_end) {  // this workgroup's chunks: publish
+          mst[c] = m;
+          gbar[c] = expf(gc + m - mn);
+          msh[c - c_first] = m;
+          msh[c - c_first + 1] = mn;
+          if (c == NC - 1) {
+            mst[NC] = mn;
+            if (m_last != nullptr) m_last[bh] = mn;
+          }
+        }
         m = mn;
       }
-      // the lane that owns the last chunk holds the final m
-      if (c_hi == NC && c_lo < NC) mst[NC] = m;
     }
   }
   __syncthreads();
 
-  // ---- phase 3: elementwise finalisation
-  for (size_t t = tid; t < Sp; t += kGateThreads) {
-    const int c = (int)(t / kChunk);
-    const float mp = mst[c], mn = mst[c + 1];
+  // elementwise finalisation of this workgroup's chunks
+  const size_t t_lo = (size_t)c_first * kChunk, t_hi = (size_t)c_end * kChunk;
+  for (size_t t = t_lo + tid; t < t_hi; t += kGateThreads) {
+    const int cl = (int)(t / kChunk) - c_first;
+    const float mp = msh[cl], mn = msh[cl + 1];
     const float b = u[t], mi = mcomb[t], a = abar[t];
     const float mc = sig_gate ? 0.f : fmaxf(b + mp, mi);
     u[t] = b - mc;
@@ -163,14 +192,14 @@ __global__ __launch_bounds__(kGateThreads) void gates_kernel(
     abar[t] = expf(a - mn);
     mcomb[t] = mc;
   }
-  if (tid == 0 && m_last != nullptr) m_last[bh] = mst[NC];
 }
 
 const char* launch_gates(const void* i, const void* f, const float* m0, const GateBufs& gb, float* m_last,
                          int B, int NH, int S, int dtype_gates, int sig_gate, hipStream_t stream) {
   const int NC = (S + kChunk - 1) / kChunk;
-  hipLaunchKernelGGL(gates_kernel, dim3(B * NH), dim3(kGateThreads), 0, stream, i, f, m0, gb, m_last, S, NC,
-                     dtype_gates, sig_gate);
+  const dim3 grid((NC + kGateChunks - 1) / kGateChunks, B * NH);
+  hipLaunchKernelGGL(gates_scan_kernel, grid, dim3(kGateThreads), 0, stream, i, f, gb, S, NC, dtype_gates, sig_gate);
+  hipLaunchKernelGGL(gates_finish_kernel, grid, dim3(kGateThreads), 0, stream, m0, gb, m_last, NC, sig_gate);
   return nullptr;
 }
 
@@ -178,35 +207,57 @@ const char* launch_gates(const void* i, const void* f, const float* m0, const Ga
 // mlstm_kernels/torch/chunkwise/triton_xl_chunk_siging/chunkwise_gates.py:72-100 in the reference):
 //   dF[t] = sigmoid(-f_t) * sum_{u >= t} (q_u.dQ_u - k_u.dK_u)     (suffix sum over the WHOLE sequence)
 //   dI[t] = k_t.dK_t   (times sigmoid(-i_t) for the sigmoid input gate)
-// One workgroup per (batch, head); every thread owns a contiguous strip, strips are combined by a
-// reverse scan over lanes and waves.
+// One workgroup per (batch, head, segment of 2048 positions), two neighbouring positions per thread (coalesced):
+// the workgroup first adds up everything behind its segment (a plain strided sum over at most S positions), then
+// scans its own segment backwards across lanes and waves.
+constexpr int kGradSeg = 2 * kGateThreads;
+
 __global__ __launch_bounds__(kGateThreads) void gate_grads_kernel(GateGradArgs a) {
   __shared__ float wtot[kGateThreads / kWave];
-  const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int S = a.S;
   const size_t Sp = (size_t)a.NC * kChunk;
   const float* qdq = a.qdq + bh * Sp;
   const float* kdk = a.kdk + bh * Sp;
-  const int R = (S + kGateThreads - 1) / kGateThreads;
-  const int lo = min(tid * R, S), hi = min(lo + R, S);
-  float tot = 0.f;
-  for (int t = lo; t < hi; ++t) tot += qdq[t] - kdk[t];
+  const int seg_lo = blockIdx.x * kGradSeg;
+  const int seg_hi = min(seg_lo + kGradSeg, S);
+  // everything behind this segment
+  float part = 0.f;
+  for (int t = seg_hi + tid; t < S; t += kGateThreads) part += qdq[t] - kdk[t];
+  part = wave_sum(part);
+  if (lane == 0) wtot[wave] = part;
+  __syncthreads();
+  float after = 0.f;
+#pragma unroll
+  for (int w = 0; w < kGateThreads / kWave; ++w) after += wtot[w];
+  __syncthreads();
+  // this segment, backwards
+  const int t0 = seg_lo + 2 * tid;
+  float kd[2], d[2];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    kd[e] = t0 + e < S ? kdk[t0 + e] : 0.f;
+    d[e] = t0 + e < S ? qdq[t0 + e] - kd[e] : 0.f;
+  }
+  const float pair = d[0] + d[1];
   auto add = [](float x, float y) { return x + y; };
-  const float rincl = wave_rev_incl_scan(tot, add);       // sum over lanes >= lane
+  const float rincl = wave_rev_incl_scan(pair, add);  // sum over lanes >= lane
   if (lane == 0) wtot[wave] = rincl;
   __syncthreads();
-  float after = rincl - tot;                              // strips of higher lanes in this wave
   for (int w = wave + 1; w < kGateThreads / kWave; ++w) after += wtot[w];
-  float run = after;
-  for (int t = hi - 1; t >= lo; --t) {
-    const size_t o = (size_t)bh * S + t;
-    const float kd = kdk[t];
-    run += qdq[t] - kd;
-    const float fv = load_scalar(a.f, o, a.dtype_gates);
-    a.dF[o] = run * (1.f / (1.f + expf(fv)));            // sigmoid(-f)
-    float di = kd;
-    if (a.sig_gate) di *= 1.f / (1.f + expf(load_scalar(a.i, o, a.dtype_gates)));
-    a.dI[o] = di;
+  float suf[2];
+  suf[1] = after + (rincl - pair) + d[1];
+  suf[0] = suf[1] + d[0];
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    if (t0 + e < S) {
+      const size_t o = (size_t)bh * S + t0 + e;
+      const float fv = load_scalar(a.f, o, a.dtype_gates);
+      a.dF[o] = suf[e] * (1.f / (1.f + expf(fv)));  // sigmoid(-f)
+      float di = kd[e];
+      if (a.sig_gate) di *= 1.f / (1.f + expf(load_scalar(a.i, o, a.dtype_gates)));
+      a.dI[o] = di;
+    }
   }
 }
 
@@ -215,7 +266,7 @@ __global__ void fill_zero_kernel(float* p, size_t n) {
 }
 
 const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream) {
-  hipLaunchKernelGGL(gate_grads_kernel, dim3(BH), dim3(kGateThreads), 0, stream, a);
+  hipLaunchKernelGGL(gate_grads_kernel, dim3((a.S + kGradSeg - 1) / kGradSeg, BH), dim3(kGateThreads), 0, stream, a);
   return nullptr;
 }
 

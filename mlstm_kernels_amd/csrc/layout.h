@@ -2,7 +2,7 @@
 //
 // Forward workspace (everything the backward re-uses lives here):
 //   gate vectors   u, w, abar, bbar, mcomb     5 x fp32 [B*NH][NC*128]
-//   per chunk      gbar, amax                  2 x fp32 [B*NH][NC]
+//   per chunk      gbar, amax, graw            3 x fp32 [B*NH][NC]
 //   stabiliser     mstates                     fp32 [B*NH][NC+1]   (index c = value before chunk c)
 //   normaliser     nstates                     fp32 [B*NH][NC][DHQK] (n before chunk c)
 //   row normaliser nrow                        fp32 [B*NH][NC*128]  max(|den|, floor), without eps
@@ -22,6 +22,7 @@ namespace mlstm {
 
 struct GateBufs {
   float *u, *w, *abar, *bbar, *mcomb, *gbar, *amax, *mstates;
+  float* graw;  // per chunk: sum of logsig(f) over the chunk (input of the scan over chunks that yields gbar)
 };
 
 struct FwWorkspace {
@@ -60,6 +61,7 @@ inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK
   w.g.gbar = (float*)take(BH * NC * 4);
   w.g.amax = (float*)take(BH * NC * 4);
   w.g.mstates = (float*)take(BH * (NC + 1) * 4);
+  w.g.graw = (float*)take(BH * NC * 4);
   w.nstates = (float*)take(BH * NC * DHQK * 4);
   w.nrow = (float*)take(BH * Sp * 4);
   w.cstates = with_states ? (uint16_t*)take(BH * NC * (size_t)DHQK * DHHV * 2) : nullptr;
