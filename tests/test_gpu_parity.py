@@ -299,6 +299,34 @@ def test_state_passing_and_exact_value_scaling_at_full_size():
     assert not torch.isnan(H.float()).any()
 
 
+def test_long_sequence_forward_backward_is_consistent_under_state_passing():
+    """S = 131072 (1024 chunks: several refills of the scan's decay table, 64 segments of the gate kernels, 64-bit
+    offsets): the second half run on its own from the carried (C, n, m) must reproduce the one-call result, outputs
+    and gradients (the gradients of the second half do not depend on the first)."""
+    exp_op, *_ = _ops()
+    B, NH, S, DQK, DHV = 1, 2, 131072, 256, 512
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    ts = [rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DHV).bfloat16(), rn(B, NH, S), 3 + rn(B, NH, S)]
+    dH = rn(B, NH, S, DHV).bfloat16()
+    full = [t.clone().requires_grad_(True) for t in ts]
+    H, (C, n, m) = exp_op(*full, return_last_states=True, chunk_size=128)
+    H.backward(dH)
+    h = S // 2
+    with torch.no_grad():
+        _, st1 = exp_op(*(t[:, :, :h].contiguous() for t in ts), return_last_states=True, chunk_size=128)
+    second = [t[:, :, h:].clone().requires_grad_(True) for t in ts]
+    H2, (C2, n2, m2) = exp_op(*second, *st1, return_last_states=True, chunk_size=128)
+    H2.backward(dH[:, :, h:].contiguous())
+    assert not torch.isnan(H.float()).any()
+    assert rel_norm(H2, H[:, :, h:]) <= 1e-3 and rel_to_scale(H2, H[:, :, h:]) <= 1e-2
+    assert_state_close(C2, C, 1e-3, "C_last")
+    assert_state_close(n2, n, 1e-3, "n_last")
+    assert (m2 - m).abs().max().item() <= 1e-4
+    for name, a_, b_ in zip(["dQ", "dK", "dV", "dI", "dF"], full, second):
+        assert rel_norm(b_.grad, a_.grad[:, :, h:]) <= 1e-3, name
+
+
 # ------------------------------------------------------------------------------------------ any sequence length in one call
 @pytest.mark.parametrize("S", [5, 77, 293, 1001])
 def test_any_sequence_length_single_call(S):
