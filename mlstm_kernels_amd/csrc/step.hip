@@ -34,6 +34,24 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
   const int tid = threadIdx.x;
   const int tx = tid % TX, ty = tid / TX;
 
+  // Small states (the cacheable variant: few workgroups per CU, nothing else to hide the prologue behind): the
+  // first batch of state rows is requested before anything else, so that the loads travel while the gates, q.n'
+  // and the LDS staging below are computed (none of which they depend on).  With a large state many workgroups
+  // per CU overlap each other's prologues and the extra live registers only cost occupancy (measured: 0.373 ms
+  // against 0.358 ms at B = 256), so the streaming variant does not do it.
+  const int col = col0 + 4 * tx;
+  const bool col_ok = col < DHHV;  // DHHV % 4 == 0 is checked on the host
+  const float* cin = c_in + (size_t)bh * DHQK * DHHV + col;
+  float* cout = c_out + (size_t)bh * DHQK * DHHV + col;
+  const bool have_first = !NONTEMPORAL && col_ok && ty + (UNROLL - 1) * TY < DHQK;
+  f32x4 cfirst[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    const f32x4* p = (const f32x4*)(cin + (size_t)(ty + u * TY) * DHHV);
+    cfirst[u] = have_first ? *p : z;
+  }
+
   const float fpre = load_scalar(fg, bh, dtype_gates);
   const float ipre = load_scalar(ig, bh, dtype_gates);
   const float m_old = m_in[bh];
@@ -65,8 +83,6 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
   const float inv_den = 1.f / (fmaxf(fabsf(qn), expf(-m_new)) + eps);
   if (blockIdx.x == 0 && tid == 0) m_out[bh] = m_new;
 
-  const int col = col0 + 4 * tx;
-  const bool col_ok = col < DHHV;  // DHHV % 4 == 0 is checked on the host
   f32x4 v4 = {0.f, 0.f, 0.f, 0.f};
   if (col_ok) {
     const size_t o = (size_t)bh * DHHV + col;
@@ -82,9 +98,17 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
   }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   if (col_ok) {
-    const float* cin = c_in + (size_t)bh * DHQK * DHHV + col;
-    float* cout = c_out + (size_t)bh * DHQK * DHHV + col;
     int r = ty;
+    if (have_first) {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int rr = r + u * TY;
+        const f32x4 o = fa * cfirst[u] + ik[rr] * v4;
+        *(f32x4*)(cout + (size_t)rr * DHHV) = o;
+        acc += qs[rr] * o;
+      }
+      r += UNROLL * TY;
+    }
     for (; r + (UNROLL - 1) * TY < DHQK; r += UNROLL * TY) {
       f32x4 c[UNROLL];
 #pragma unroll
@@ -145,18 +169,21 @@ const char* launch_step(const void* q, const void* k, const void* v, const void*
   if (B <= 0 || NH <= 0 || DHQK <= 0 || DHHV <= 0) return "mlstm_hip_step: non-positive dimension";
   if (DHHV % 4 != 0) return "mlstm_hip_step: DHHV must be a multiple of 4";
   if ((long long)B * NH > 65535) return "mlstm_hip_step: B*NH exceeds 65535";
-  // Tile shapes from a sweep on MI355X (B = 16/64/256, NH = 8, 256 x 512 state): 256-column slices with 8 row
-  // groups are fastest; a state that fits the 256 MB memory-side cache is best left cacheable (it is re-read
-  // by the next step), a larger one streams past the caches with non-temporal accesses and deeper unrolling.
+  // Tile shapes from a sweep on MI355X (B = 16/64/256, NH = 8, 256 x 512 state).  A state larger than the 256 MB
+  // memory-side cache streams past the caches with non-temporal accesses: 256-column slices, 8 row groups, 16 rows
+  // in flight per lane.  A smaller one is best left cacheable (it is re-read by the next step) and has few
+  // workgroups per CU: 128-column slices with 16 row groups, the first 16 rows per lane requested before the
+  // prologue.  The crossover was measured between a 268 MB state (cacheable 79 us, streaming 90 us) and a 403 MB
+  // state (156 us against 133 us).
   const size_t state_bytes = (size_t)B * NH * DHQK * DHHV * sizeof(float);
-  const bool stream_past_cache = state_bytes > ((size_t)200 << 20);
+  const bool stream_past_cache = state_bytes > ((size_t)320 << 20);
 #define MLSTM_STEP_ARGS q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps, dtype_qkv, dtype_gates, stream
   if (DHHV % 256 == 0) {
     if (stream_past_cache) return launch_step_t<256, 8, 16, true>(MLSTM_STEP_ARGS);
-    return launch_step_t<256, 8, 8, false>(MLSTM_STEP_ARGS);
+    return launch_step_t<128, 16, 16, false>(MLSTM_STEP_ARGS);
   }
   if (stream_past_cache) return launch_step_t<128, 8, 8, true>(MLSTM_STEP_ARGS);
-  return launch_step_t<128, 8, 8, false>(MLSTM_STEP_ARGS);
+  return launch_step_t<128, 16, 16, false>(MLSTM_STEP_ARGS);
 #undef MLSTM_STEP_ARGS
 }
 #endif
