@@ -386,7 +386,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
   MLSTM_PTICK(5)
 #ifdef MLSTM_PAR_TIMING
   if (blk.y == a.NC / 2 && blk.z == 0 && lane == 0)
-    for (int p = 0; p < 6; ++p) a.timing[(blk.x * 4 + (wave & 3)) * 8 + p] = tph[p];
+    for (int p = 0; p < 6; ++p) a.timing[((blk.x + (IS_DQ ? 0 : 2)) * 4 + (wave & 3)) * 8 + p] = tph[p];
   if (tid == 0) {
     const size_t wg = ((size_t)blk.z * a.NC + blk.y) * 2 + blk.x + (IS_DQ ? 0 : 8192);
     a.timing[64 + wg * 2] = tstart;
