@@ -21,7 +21,9 @@
 //
 // Measured on MI355X at B=4, S=16384, 256/512 and not kept: eight waves of 32 head-dim rows per workgroup (four
 // waves per SIMD; 0.99 ms against 0.97 ms for the pair launch); dV's workgroups in the same launch as well (1.56 ms
-// against 1.52 ms for dV followed by the pair launch: they stream the shared operands in another order).
+// against 1.52 ms for dV followed by the pair launch: they stream the shared operands in another order); the Xo score
+// operands fetched straight from global memory in fragment layout instead of through LDS (1.03 against 0.98 ms: 32-byte
+// row pieces per lane pair are a poor access pattern, the LDS detour is cheaper).
 #include "common.h"
 #include "kernels.h"
 
