@@ -34,7 +34,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
   constexpr int NWAVE = MT / 64;    // each wave owns 64 head-dim rows = 2 MFMA row blocks
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;       // P stored as Ps[n][o]
-  constexpr int XS = 32 + 8;        // value-column slab row stride (32 columns per slab)
+  constexpr int XS = 64 + 8;        // row stride of the Xn / Xo slabs (64 value columns: two state slabs)
   constexpr int ZS = MT + 16;       // pass-2 slab row stride
   constexpr int OS = MT + 8;        // output staging row stride
   constexpr int NDT = MT / 16;      // 16-row state fragments per 32 value columns inside the tile
@@ -106,48 +106,57 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
       for (int i = 0; i < 16; ++i) sacc[k][nb][i] = 0.f;
   const int m_wave = wave * 64;
 
-  // ---- pass 1 over the value columns, 32 per slab, register-prefetched one slab ahead
+  // ---- pass 1 over the value columns
   {
     const size_t ND = DHQK / 16, NW = DHHV / 32;
     const u32x4* st = (const u32x4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
     constexpr int CV = NDT * 64 / NTH;      // state-fragment vectors per thread per slab
-    constexpr int NV = 64 * 4 / NTH;        // Xn vectors per thread per slab
-    constexpr int OV = 128 * 4 / NTH;       // Xo vectors per thread per slab
+    // The state fragments come in slabs of 32 value columns, two slabs in flight in registers.  The Xn / Xo rows are
+    // fetched 64 columns at a time (one fetch serves two state slabs): 128 contiguous bytes per row and load
+    // instruction instead of 64.
+    constexpr int NV = 64 * 8 / NTH;        // Xn vectors per thread per pair of slabs
+    constexpr int OV = 128 * 8 / NTH;       // Xo vectors per thread per pair of slabs
     u32x4 cregA[CV], cregB[CV];
-    uint4 nregA[NV], oregA[OV], nregB[NV], oregB[OV];
+    uint4 nreg[NV], oreg[OV];
     // (macros, not lambdas: with the arrays captured by reference the compiler kept them in scratch memory)
-#define MLSTM_LOAD_SLAB(slab_, creg, nreg, oreg)                                                                     \
+#define MLSTM_LOAD_C(slab_, creg)                                                                                    \
   {                                                                                                                  \
     _Pragma("unroll") for (int v = 0; v < CV; ++v)                                                                   \
         creg[v] = st[((size_t)(slab_) * ND + d_tile / 16) * 64 + tid + v * NTH];                                     \
+  }
+#define MLSTM_LOAD_X(pair_)                                                                                          \
+  {                                                                                                                  \
     _Pragma("unroll") for (int v = 0; v < NV; ++v) {                                                                 \
       const int idx = tid + v * NTH;                                                                                 \
-      const int t = t_base + n0 + (idx >> 2);                                                                        \
-      nreg[v] = t < S ? *(const uint4*)(Xn_g + (size_t)t * DHHV + (slab_) * 32 + (idx & 3) * 8) : make_uint4(0, 0, 0, 0); \
+      const int t = t_base + n0 + (idx >> 3);                                                                        \
+      nreg[v] = t < S ? *(const uint4*)(Xn_g + (size_t)t * DHHV + (pair_) * 64 + (idx & 7) * 8) : make_uint4(0, 0, 0, 0); \
     }                                                                                                                \
     _Pragma("unroll") for (int v = 0; v < OV; ++v) {                                                                 \
       const int idx = tid + v * NTH;                                                                                 \
-      const int j = idx >> 2;                                                                                        \
+      const int j = idx >> 3;                                                                                        \
       const int t = t_base + j;                                                                                      \
       const bool live = j >= 32 * ob_lo && j < 32 * ob_hi && t < S;                                                  \
-      oreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHHV + (slab_) * 32 + (idx & 3) * 8) : make_uint4(0, 0, 0, 0); \
+      oreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHHV + (pair_) * 64 + (idx & 7) * 8) : make_uint4(0, 0, 0, 0); \
     }                                                                                                                \
   }
     // lanes 32..63 of every state fragment are stored 4 slots off so that the two lane halves a transposing read
     // touches together fall on different LDS banks
-#define MLSTM_STORE_SLAB(creg, nreg, oreg)                                                                           \
+#define MLSTM_STORE_C(creg)                                                                                          \
   {                                                                                                                  \
     _Pragma("unroll") for (int v = 0; v < CV; ++v) {                                                                 \
       const int idx = tid + v * NTH;                                                                                 \
       ((u32x4*)Cf)[idx ^ (((idx >> 5) & 1) << 2)] = creg[v];                                                         \
     }                                                                                                                \
+  }
+#define MLSTM_STORE_X                                                                                                \
+  {                                                                                                                  \
     _Pragma("unroll") for (int v = 0; v < NV; ++v) {                                                                 \
       const int idx = tid + v * NTH;                                                                                 \
-      *(uint4*)(Xn + (idx >> 2) * XS + (idx & 3) * 8) = nreg[v];                                                     \
+      *(uint4*)(Xn + (idx >> 3) * XS + (idx & 7) * 8) = nreg[v];                                                     \
     }                                                                                                                \
     _Pragma("unroll") for (int v = 0; v < OV; ++v) {                                                                 \
       const int idx = tid + v * NTH;                                                                                 \
-      *(uint4*)(Xo + (idx >> 2) * XS + (idx & 3) * 8) = oreg[v];                                                     \
+      *(uint4*)(Xo + (idx >> 3) * XS + (idx & 7) * 8) = oreg[v];                                                     \
     }                                                                                                                \
   }
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
@@ -156,12 +165,13 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
     const int d_grp = i16 & 3;
     const int h_src = d_grp & 1, a_src = d_grp >> 1;
     const int nslab = DHHV / 32;  // even: DHHV is a multiple of 64
-    auto multiply_slab = [&]() {
+    auto multiply_slab = [&](const int sub) {  // sub = which half of the staged Xn / Xo columns
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         Frag B[2];
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Xn + (32 * nb + r) * XS + 16 * ks + 8 * h);
+        for (int nb = 0; nb < 2; ++nb)
+          B[nb].u = *(const uint4*)(Xn + (32 * nb + r) * XS + 32 * sub + 16 * ks + 8 * h);
         // inter-chunk product: A = State[d][w]
         {
           Frag A[2];
@@ -191,33 +201,38 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
           const int ob = ob_lo + wave + k * NWAVE;
           const int obc = ob < 4 ? ob : 3;
           Frag A;
-          A.u = *(const uint4*)(Xo + (32 * obc + r) * XS + 16 * ks + 8 * h);
+          A.u = *(const uint4*)(Xo + (32 * obc + r) * XS + 32 * sub + 16 * ks + 8 * h);
 #pragma unroll
           for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
         }
       }
     };
-    // two slabs are in flight in registers while a third is multiplied: one memory round trip spans two slab
-    // periods.  The prefetches are unconditional (the last iterations re-fetch the last slab): a conditional
-    // prefetch makes the compiler keep the prefetch registers in scratch memory across the loop back-edge.
-    MLSTM_LOAD_SLAB(0, cregA, nregA, oregA)
-    MLSTM_LOAD_SLAB(1, cregB, nregB, oregB)
+    // two state slabs and one Xn / Xo pair are in flight in registers while a slab is multiplied: one memory round
+    // trip spans two slab periods.  The prefetches are unconditional (the last iterations re-fetch the last slab): a
+    // conditional prefetch makes the compiler keep the prefetch registers in scratch memory across the loop back-edge.
+    MLSTM_LOAD_C(0, cregA)
+    MLSTM_LOAD_X(0)
+    MLSTM_LOAD_C(1, cregB)
     MLSTM_PTICK(0)
     for (int slab = 0; slab < nslab; slab += 2) {
       __syncthreads();
-      MLSTM_STORE_SLAB(cregA, nregA, oregA)
+      MLSTM_STORE_C(cregA)
+      MLSTM_STORE_X
       __syncthreads();
-      MLSTM_LOAD_SLAB(slab + 2 < nslab ? slab + 2 : nslab - 1, cregA, nregA, oregA)
-      multiply_slab();
+      MLSTM_LOAD_C(slab + 2 < nslab ? slab + 2 : nslab - 1, cregA)
+      MLSTM_LOAD_X(slab + 2 < nslab ? slab / 2 + 1 : slab / 2)
+      multiply_slab(0);
       __syncthreads();
-      MLSTM_STORE_SLAB(cregB, nregB, oregB)
+      MLSTM_STORE_C(cregB)
       __syncthreads();
-      MLSTM_LOAD_SLAB(slab + 3 < nslab ? slab + 3 : nslab - 1, cregB, nregB, oregB)
-      multiply_slab();
+      MLSTM_LOAD_C(slab + 3 < nslab ? slab + 3 : nslab - 1, cregB)
+      multiply_slab(1);
     }
   }
-#undef MLSTM_STORE_SLAB
-#undef MLSTM_LOAD_SLAB
+#undef MLSTM_STORE_C
+#undef MLSTM_STORE_X
+#undef MLSTM_LOAD_C
+#undef MLSTM_LOAD_X
   MLSTM_PTICK(1)
   // column scale of the inter-chunk part
 #pragma unroll
@@ -419,7 +434,7 @@ __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(M
 template <int MT>
 static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t stream) {
   constexpr int CF = (MT / 16) * 64 * 8;
-  constexpr int sa = CF + 64 * 40 + 128 * 40, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
+  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
   constexpr int sab = sa > sb ? sa : sb;
   constexpr int stage = sab > sc ? sab : sc;
   const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;
