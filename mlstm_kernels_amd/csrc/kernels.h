@@ -24,6 +24,9 @@ struct ScanArgs {
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
   int backward;
+#ifdef MLSTM_SCAN_TIMING
+  unsigned long long* timing;  // one-off timing builds
+#endif
 };
 
 struct ParHvArgs {

@@ -59,6 +59,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   uint16_t* Yl = Yh + PS * YS;
   float* npart = (float*)(Yl + (HILO ? PS * YS : 0));  // [XROWS][RT] partial sums of the n update
   float* gl = npart + XROWS * RT;                       // [kGBlock] decay factors of the next chunks, in scan order
+  float* scl = gl + kGBlock;                            // [2][128] row scales of the chunk being staged / the next one
 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -106,9 +107,22 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   const uint16_t* Yg = a.Y + (size_t)bh * S * DHHV + w_tile;
 
   uint4 xr[XV], yr[YV];
-  float xsc[XV], ysc[YV], ynr[YV];
-  // The prefetch only LOADS (raw scale factors included): any arithmetic on a loaded value here would make the
-  // wave wait for the whole batch of loads before it starts the matrix work they are meant to overlap with.
+  // Row scales (forward: abar_j; backward: bbar_t / sqrt(DHQK) / (nrow_t + eps)) go through a table in LDS instead of
+  // one 4-byte load per staged vector: every thread fetches the factor of ONE row two chunks ahead (a single load
+  // instruction per wave and chunk), the table entry is written while the chunk before it is staged.  The vector
+  // memory path of the CU (64 bytes per clock for loads, stores and their address processing) is what the scan
+  // queues on, so its instruction count matters.
+  const int srow = tid & (kChunk - 1);
+  const float* const nrow_or_dummy = a.nrow != nullptr ? a.nrow : a.scale_a;
+  float s_raw = 0.f, s_nrm = 1.f;
+  auto load_scales = [&](int c) {
+    const int cc = min(max(c, 0), NC - 1);
+    const int t = cc * kChunk + srow;
+    s_raw = a.scale_a[bh * Sp + t];
+    s_nrm = nrow_or_dummy[bh * Sp + t];
+  };
+  // The prefetch only LOADS: any arithmetic on a loaded value here would make the wave wait for the whole batch of
+  // loads before it starts the matrix work they are meant to overlap with.
   auto prefetch = [&](int c, int piece) {
 #pragma unroll
     for (int v = 0; v < XV; ++v) {
@@ -116,7 +130,6 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       const int j = idx / (RT / 8), cv = idx % (RT / 8);
       const int t = c * kChunk + piece * PS + j;
       xr[v] = t < S ? *(const uint4*)(Xg + (size_t)t * DHQK + cv * 8) : make_uint4(0, 0, 0, 0);
-      if (do_n) xsc[v] = t < S ? a.scale_a[bh * Sp + t] : 0.f;
     }
 #pragma unroll
     for (int v = 0; v < YV; ++v) {
@@ -124,12 +137,27 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
       const int t = c * kChunk + piece * PS + j;
       yr[v] = t < S ? *(const uint4*)(Yg + (size_t)t * DHHV + cv * 8) : make_uint4(0, 0, 0, 0);
-      ysc[v] = t < S ? a.scale_a[bh * Sp + t] : 0.f;
-      if (a.backward && a.nrow != nullptr) ynr[v] = a.nrow[bh * Sp + t];
     }
   };
 
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
+#ifdef MLSTM_SCAN_TIMING
+  unsigned long long tph[5] = {0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
+#define MLSTM_STICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
+#else
+#define MLSTM_STICK(p_)
+#endif
+  // row scales of the first chunk straight into the table, those of the second chunk into the prefetch register
+  {
+    const int t = c_first * kChunk + srow;
+    float sc0 = t < S ? a.scale_a[bh * Sp + t] : 0.f;
+    if (a.backward) {
+      sc0 *= a.qk_scale;
+      if (a.nrow != nullptr) sc0 /= (a.nrow[bh * Sp + t] + a.eps);
+    }
+    if (tid < kChunk) scl[srow] = sc0;
+  }
+  load_scales(NC > 1 ? c_first + c_step : c_first);
   prefetch(c_first, 0);
   for (int hit = 0; hit < NC * NP; ++hit) {
     const int it = hit / NP, piece = hit % NP;
@@ -143,6 +171,17 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       // visible after the barrier that follows the staging below
     }
     // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split); partial sums of sum_j abar_j k_j
+    const float* scur = scl + (it & 1) * kChunk + piece * PS;  // written while the previous chunk was staged
+    if (piece == 0 && tid < kChunk) {
+      // the next chunk's row scales (fetched two chunks ahead) into the other half of the table
+      const int t = (c + c_step) * kChunk + srow;
+      float sn = (it + 1 < NC && t < S) ? s_raw : 0.f;
+      if (a.backward) {
+        sn *= a.qk_scale;
+        if (a.nrow != nullptr) sn /= (s_nrm + a.eps);
+      }
+      scl[((it + 1) & 1) * kChunk + srow] = sn;
+    }
     float np[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int v = 0; v < XV; ++v) {
@@ -151,10 +190,11 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       *(uint4*)(Xs + j * XS + cv * 8) = xr[v];
       if (do_n) {
         const uint32_t in[4] = {xr[v].x, xr[v].y, xr[v].z, xr[v].w};
+        const float xsc = scur[j];
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-          np[2 * p] += xsc[v] * __uint_as_float(in[p] << 16);
-          np[2 * p + 1] += xsc[v] * __uint_as_float(in[p] & 0xffff0000u);
+          np[2 * p] += xsc * __uint_as_float(in[p] << 16);
+          np[2 * p + 1] += xsc * __uint_as_float(in[p] & 0xffff0000u);
         }
       }
     }
@@ -170,11 +210,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       const int j = idx / (WT / 8), cv = idx % (WT / 8);
       const uint32_t in[4] = {yr[v].x, yr[v].y, yr[v].z, yr[v].w};
       uint32_t hi[4], lo[4];
-      float sc = ysc[v];
-      if (a.backward) {
-        sc *= a.qk_scale;
-        if (a.nrow != nullptr) sc /= (ynr[v] + a.eps);
-      }
+      const float sc = scur[j];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
         const float e0 = __uint_as_float(in[p] << 16) * sc;
@@ -185,8 +221,11 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       *(uint4*)(Yh + j * YS + cv * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
       if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     }
+    MLSTM_STICK(0)
     __syncthreads();
+    MLSTM_STICK(1)
     if (hit + 1 < NC * NP) prefetch(piece + 1 < NP ? c : c + c_step, piece + 1 < NP ? piece + 1 : 0);
+    if (piece == 0) load_scales(c + 2 * c_step);
 
     // ---- emit the state before this chunk's update as bf16 operand fragments
     if (piece == 0) {
@@ -208,6 +247,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
           }
         }
     }
+    MLSTM_STICK(2)
     // ---- decay (once per chunk), then accumulate X^T (scale . Y) over the positions of this piece
     const float g = piece == 0 ? gl[it & (kGBlock - 1)] : 1.f;
     if (piece == 0) {
@@ -254,8 +294,14 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       for (int g2 = 0; g2 < XROWS; ++g2) s += npart[g2 * RT + tid];
       nval = g * nval + s;
     }
+    MLSTM_STICK(3)
     __syncthreads();
+    MLSTM_STICK(4)
   }
+#ifdef MLSTM_SCAN_TIMING
+  if (bx == 0 && by == 0 && bz == 0 && lane == 0)
+    for (int p = 0; p < 5; ++p) a.timing[wave * 8 + p] = tph[p];
+#endif
 
   if (a.final_out != nullptr) {
 #pragma unroll
@@ -282,7 +328,7 @@ static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) 
   constexpr int XROWS = NT / (RT / 8);
   constexpr int PS = 128;
   const size_t smem = (size_t)PS * (RT + 16) * 2 + (size_t)PS * (WT + 16) * 2 * (HILO ? 2 : 1) +
-                      (size_t)(XROWS * RT + kGBlock) * 4;
+                      (size_t)(XROWS * RT + kGBlock + 2 * kChunk) * 4;
   if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS, WCOLS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "scan: cannot raise the dynamic LDS limit";
