@@ -62,7 +62,7 @@ ALG_BYTES = {
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload (calibrated against a
 # copy kernel of known size; summary in profiles/tfla_fwbw_B4_S16384__step_B256__pmc_hbm_traffic.md)
 MEASURED_HBM_BYTES = {
-    "scan_fw": 2012e6, "par_h": 2800e6, "scan_bw": 1962e6, "par_dv": 2920e6, "par_dqdk": 4336e6,
+    "scan_fw": 2242e6, "par_h": 2807e6, "scan_bw": 1884e6, "par_dv": 2921e6, "par_dqdk": 4324e6,
     "step": 2163e6,
 }
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
