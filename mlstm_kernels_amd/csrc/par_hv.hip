@@ -386,7 +386,8 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
       for (int idx = tid; idx < 32 * vec_per_row; idx += NTH) {
         const int j = idx / vec_per_row, cv = idx % vec_per_row;
         const int t = t_base + n0 + 32 * nb + j;
-        if (t < S) *(uint4*)(Og + (size_t)t * DHHV + cv * 8) = *(const uint4*)(Ts + j * HS + cv * 8);
+        // non-temporal: nobody in this launch reads the output, it should not evict shared operands from the L2
+        if (t < S) __builtin_nontemporal_store(*(const u32x4*)(Ts + j * HS + cv * 8), (u32x4*)(Og + (size_t)t * DHHV + cv * 8));
       }
     }
   }

@@ -397,7 +397,8 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
     for (int idx = tid; idx < 64 * vec_per_row; idx += NTH) {
       const int j = idx / vec_per_row, cv = idx % vec_per_row;
       const int t = t_base + n0 + j;
-      if (t < S) *(uint4*)(Og + (size_t)t * DHQK + cv * 8) = *(const uint4*)(Os + j * OS + cv * 8);
+      // non-temporal: nobody in this launch reads the output, it should not evict shared operands from the L2
+      if (t < S) __builtin_nontemporal_store(*(const u32x4*)(Os + j * OS + cv * 8), (u32x4*)(Og + (size_t)t * DHQK + cv * 8));
     }
   }
   MLSTM_PTICK(5)

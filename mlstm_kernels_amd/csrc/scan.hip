@@ -243,7 +243,10 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
             f.y = pack_bf16x2(acc[db][wb][8 * half + 2], acc[db][wb][8 * half + 3]);
             f.z = pack_bf16x2(acc[db][wb][8 * half + 4], acc[db][wb][8 * half + 5]);
             f.w = pack_bf16x2(acc[db][wb][8 * half + 6], acc[db][wb][8 * half + 7]);
-            st[(W32 * ND + D16 + half) * 64 + lane] = f;
+            // non-temporal: the fragments are read by a later kernel; kept out of the L2 they do not evict the K/V
+            // rows the tiles of a head share
+            const u32x4 fv = {f.x, f.y, f.z, f.w};
+            __builtin_nontemporal_store(fv, (u32x4*)(st + (W32 * ND + D16 + half) * 64 + lane));
           }
         }
     }
