@@ -62,7 +62,7 @@ ALG_BYTES = {
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload (calibrated against a
 # copy kernel of known size; summary in profiles/tfla_fwbw_B4_S16384__step_B256__pmc_hbm_traffic.md)
 MEASURED_HBM_BYTES = {
-    "scan_fw": 2242e6, "par_h": 2807e6, "scan_bw": 1884e6, "par_dv": 2921e6, "par_dqdk": 4324e6,
+    "scan_fw": 2122e6, "par_h": 2763e6, "scan_bw": 1883e6, "par_dv": 2890e6, "par_dqdk": 4319e6,
     "step": 2163e6,
 }
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
