@@ -48,7 +48,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;      // score matrix row stride: P stored as Ps[n][o]
   constexpr int KS = 64 + 8;       // slab row stride of the streamed score operand
-  constexpr int VS = WT + 16;      // slab row stride of the streamed value-side operand
+  constexpr int VS = WT + 32;      // slab row stride of the streamed value-side operand (rows 64 bytes apart in the banks)
   constexpr int HS = WT + 8;       // output staging row stride
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   const int QS = DHQK + 8;
@@ -409,7 +409,7 @@ template <int WT, bool IS_DV, int PD, int MW>
 static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
   const int QS = a.DHQK + 8;
   const size_t n_region = (size_t)64 * QS;
-  const size_t t_region = (128 * 72 > 32 * (WT + 16)) ? 128 * 72 : 32 * (WT + 16);
+  const size_t t_region = (128 * 72 > 32 * (WT + 32)) ? 128 * 72 : 32 * (WT + 32);
   const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + 8 * 32 + a.DHQK) * 4;
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
   if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, IS_DV, PD, MW>, hipFuncAttributeMaxDynamicSharedMemorySize,

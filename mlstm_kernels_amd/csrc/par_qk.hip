@@ -35,7 +35,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
   constexpr int NTH = 64 * NWAVE;
   constexpr int PS = 128 + 8;       // P stored as Ps[n][o]
   constexpr int XS = 64 + 8;        // row stride of the Xn / Xo slabs (64 value columns: two state slabs)
-  constexpr int ZS = MT + 16;       // pass-2 slab row stride
+  constexpr int ZS = MT + 32;       // pass-2 slab row stride (rows 64 bytes apart in the banks)
   constexpr int OS = MT + 8;        // output staging row stride
   constexpr int NDT = MT / 16;      // 16-row state fragments per 32 value columns inside the tile
   constexpr int CF = NDT * 64 * 8;  // elements of the staged state fragments per 32-column slab
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(M
 template <int MT>
 static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t stream) {
   constexpr int CF = (MT / 16) * 64 * 8;
-  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 32 * (MT + 16);
+  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 32 * (MT + 32);
   constexpr int sab = sa > sb ? sa : sb;
   constexpr int stage = sab > sc ? sab : sc;
   const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;

@@ -46,8 +46,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   constexpr int WC = WT / WCOLS;
   constexpr int NBW = WCOLS / 32;  // 32-column accumulator blocks per wave
   constexpr int NT = 64 * (RT / 64) * WC;
-  constexpr int XS = RT + 16;  // LDS row strides (elements); +16 keeps 4 consecutive rows on distinct banks
-  constexpr int YS = WT + 16;
+  constexpr int XS = RT + 32;  // LDS row strides (elements): consecutive rows start 16 banks (64 bytes) apart
+  constexpr int YS = WT + 32;
   constexpr int XV = PS * RT / 8 / NT;   // 16-byte vectors per thread per piece
   constexpr int YV = PS * WT / 8 / NT;
   constexpr int NP = kChunk / PS;        // pieces per chunk
@@ -330,7 +330,7 @@ static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) 
   constexpr int NT = 64 * (RT / 64) * (WT / WCOLS);
   constexpr int XROWS = NT / (RT / 8);
   constexpr int PS = 128;
-  const size_t smem = (size_t)PS * (RT + 16) * 2 + (size_t)PS * (WT + 16) * 2 * (HILO ? 2 : 1) +
+  const size_t smem = (size_t)PS * (RT + 32) * 2 + (size_t)PS * (WT + 32) * 2 * (HILO ? 2 : 1) +
                       (size_t)(XROWS * RT + kGBlock + 2 * kChunk) * 4;
   if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS, WCOLS>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
