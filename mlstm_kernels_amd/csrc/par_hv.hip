@@ -64,6 +64,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   float* inv = cs + 64;                 // forward: [64] 1/(nmax + eps); dV: [128] rho_t of the chunk
   float* rows = inv + 128;              // [8][32] partial row sums of Sbar per score unit (forward)
   float* nperm = rows + 8 * 32;         // [DHQK] n_prev in fragment order (forward)
+  float* mcs = nperm + DHQK;            // [64] combined stabiliser of this workgroup's positions (forward)
 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -145,8 +146,12 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
     }
     for (int idx = tid; idx < 64; idx += NTH)
       cs[idx] = IS_DV ? a.g.abar[gofs + n0 + idx] : a.g.bbar[gofs + n0 + idx] * a.qk_scale;
-    if (!IS_DV)
+    if (!IS_DV) {
       for (int d = tid; d < DHQK; d += NTH) nperm[perm16(d)] = a.nstates[((size_t)bh * NC + c) * DHQK + d];
+      // fetched with everything else: read from global memory in the denominator phase, the stabiliser costs that
+      // phase a whole trip to memory
+      for (int idx = tid; idx < 64; idx += NTH) mcs[idx] = a.g.mcomb[gofs + n0 + idx];
+    }
   }
 
   MLSTM_PTICK(0)
@@ -265,7 +270,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         float den = cs[t] * dot;
 #pragma unroll
         for (int ob4 = 0; ob4 < 4; ++ob4) den += rows[(2 * ob4 + (t >> 5)) * 32 + (t & 31)];
-        const float mc = a.g.mcomb[gofs + n0 + t];
+        const float mc = mcs[t];
         const float floor_v = a.sig_gate ? 1.f : __expf(-mc);
         nmax = fmaxf(fabsf(den), floor_v);
         iv = 1.f / (nmax + a.eps);
@@ -276,7 +281,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         const int tg = t_base + n0 + t;
         if (tg < S) {
           if (a.n_out != nullptr) a.n_out[(size_t)bh * S + tg] = nmax;
-          if (a.m_out != nullptr) a.m_out[(size_t)bh * S + tg] = a.g.mcomb[gofs + n0 + t];
+          if (a.m_out != nullptr) a.m_out[(size_t)bh * S + tg] = mcs[t];
         }
       }
     }
@@ -410,7 +415,7 @@ static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stre
   const int QS = a.DHQK + 8;
   const size_t n_region = (size_t)64 * QS;
   const size_t t_region = (128 * 72 > 32 * (WT + 32)) ? 128 * 72 : 32 * (WT + 32);
-  const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + 8 * 32 + a.DHQK) * 4;
+  const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + 8 * 32 + a.DHQK + 64) * 4;
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
   if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, IS_DV, PD, MW>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
