@@ -34,6 +34,7 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 //   four waves, half-chunk pieces so that the forward fits twice per CU          0.66 / 0.55
 //   eight waves per tile (64 x 32 per wave), one workgroup per CU                0.46 / 0.41   <- used
 //   eight waves, two workgroups per CU (128 registers per lane)                  -    / 0.45
+//   n recurrence shared out among the column tiles by lane masks / run by every column tile    0.51 / -    (0.48 used)
 // What pays is a second instruction stream per SIMD inside the same workgroup: the phases of a chunk (staging,
 // state emission, matrix work) are serial per wave, and two waves per SIMD overlap one's LDS and conversion
 // latencies with the other's matrix instructions.
