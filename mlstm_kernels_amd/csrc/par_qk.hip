@@ -44,7 +44,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
   // stage region: [state frags | Xn slab | Xo slab], later pass-2 slabs, later the output staging tile
   constexpr int stage_elems_a = CF + 64 * XS + 128 * XS;
   constexpr int stage_elems_b = 64 * OS;
-  constexpr int stage_elems_c = 32 * ZS;
+  constexpr int stage_elems_c = 64 * ZS;
   constexpr int stage_ab = stage_elems_a > stage_elems_b ? stage_elems_a : stage_elems_b;
   constexpr int stage_elems = stage_ab > stage_elems_c ? stage_ab : stage_elems_c;
   uint16_t* Cf = (uint16_t*)smem_raw;
@@ -241,8 +241,9 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= sc;
   }
-  // first pass-2 slab into registers while the score matrix is gated
-  constexpr int ZV = 32 * (MT / 8) / NTH;
+  // first pass-2 slab (64 positions: two score blocks; the live range is always an even number of blocks) into
+  // registers while the score matrix is gated
+  constexpr int ZV = 64 * (MT / 8) / NTH;
   uint4 zreg[ZV];
   auto load_zslab = [&](int ob) {
 #pragma unroll
@@ -309,7 +310,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
     uint16_t* Zs = Cf;
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
-    for (int ob = ob_lo; ob < ob_hi; ++ob) {
+    for (int ob = ob_lo; ob < ob_hi; ob += 2) {
       __syncthreads();  // first pass: P written and pass-1 slabs consumed
 #pragma unroll
       for (int v = 0; v < ZV; ++v) {
@@ -317,9 +318,9 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
         *(uint4*)(Zs + (idx / (MT / 8)) * ZS + (idx % (MT / 8)) * 8) = zreg[v];
       }
       __syncthreads();
-      if (ob + 1 < ob_hi) load_zslab(ob + 1);
+      if (ob + 2 < ob_hi) load_zslab(ob + 2);
 #pragma unroll
-      for (int jl = 0; jl < 2; ++jl) {
+      for (int jl = 0; jl < 4; ++jl) {
         Frag A[2], B[2];
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) {
@@ -435,7 +436,7 @@ __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(M
 template <int MT>
 static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t stream) {
   constexpr int CF = (MT / 16) * 64 * 8;
-  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 32 * (MT + 32);
+  constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 64 * (MT + 32);
   constexpr int sab = sa > sb ? sa : sb;
   constexpr int stage = sab > sc ? sab : sc;
   const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(3 * 128 + 64 + (MT / 64) * 64) * 4;
