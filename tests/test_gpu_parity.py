@@ -255,6 +255,8 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     dict(B=1, NH=2, S=400, DQK=128, DHV=64, L=16, init=True, dcl=True, seed=2),   # ragged tail, initial state
     dict(B=1, NH=2, S=256, DQK=128, DHV=128, siging=True, init=True, seed=3),
     dict(B=1, NH=2, S=256, DQK=256, DHV=64, siging=True, normalize=False, seed=4),
+    dict(B=1, NH=2, S=384, DQK=192, DHV=320, init=True, seed=5),   # head dimensions that are multiples of 64 only
+    dict(B=1, NH=1, S=256, DQK=320, DHV=192, dcl=True, seed=6),
 ])
 def test_chunkwise_fwbw_small(kw):
     _fwbw_case(**kw)
