@@ -50,7 +50,11 @@ def d64(t):
 
 
 # ------------------------------------------------------------------------------------------ decode step
-@pytest.mark.parametrize("B,NH,DQK,DHV", [(2, 2, 64, 128), (3, 4, 256, 512), (1, 1, 128, 192)])
+@pytest.mark.parametrize("B,NH,DQK,DHV", [
+    (2, 2, 64, 128), (3, 4, 256, 512), (1, 1, 128, 192),
+    (3, 2, 96, 100), (1, 1, 48, 36), (5, 2, 130, 260),   # odd head dimensions: partial slices, ragged row batches
+    (40, 8, 256, 512),                                    # 168 MB of state: the cacheable variant at a larger batch
+])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_step_parity(B, NH, DQK, DHV, dtype):
     *_, step, _ = _ops()
