@@ -12,7 +12,7 @@
  *   - Return value 0 = success; anything else = failure, message via mlstm_hip_last_error().
  *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1.  gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp),
  *     MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
- *   - Supported shapes: DHQK % 64 == 0, DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
+ *   - Supported shapes: DHQK % 64 == 0 (at most 896), DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
  *
  * Each entry point names the reference interface it replaces (paths relative to the reference checkout).
  */
@@ -48,20 +48,29 @@ int mlstm_hip_profile_read(int index, char* name, size_t name_cap, float* total_
 const char* mlstm_hip_last_error(void);
 
 /*
- * Kernel selection for the value-column side of the chunkwise passes (H forward, dV backward).  A tuning knob with
- * no counterpart in the reference (its Triton kernels are always the two-kernel form, recurrent_fw_C followed by
- * parallel_fw_Hintra: mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:20-136).
+ * Per-call tuning options of the chunkwise entry points (no state is kept between calls).
+ *
+ * path: kernel selection for the value-column side of the passes (H forward, dV backward).  No counterpart in the
+ * reference, whose Triton kernels are always the two-kernel form, recurrent_fw_C followed by parallel_fw_Hintra
+ * (mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:20-136).
  *   MLSTM_PATH_AUTO  : the faster one for the shape as measured on MI355X (today: split for every shape)
  *   MLSTM_PATH_SPLIT : state scan + chunk-parallel kernel over materialised chunk states
- *   MLSTM_PATH_FUSED : one sequential kernel per pass, state slice resident in registers (falls back to split
- *                      for head dimensions it does not support)
- * Process-wide; returns the previous setting.  Results of the two paths agree within the rounding of bf16 operands.
- * A forward workspace sized under one setting must be used under the same setting.
+ *   MLSTM_PATH_FUSED : one sequential kernel per pass, state slice resident in registers (DHQK = 128 or 256 only:
+ *                      other head dimensions are rejected)
+ *
+ * state_stride: a chunk state (DHQK x DHHV bf16 per chunk of 128 positions and head) is kept every state_stride
+ * chunks; chunks in between reach back to the nearest kept state through additional score blocks.  Replaces the
+ * reference's chunk_size_inter / chunk_size_intra pair with save_states_every_nth_chunk =
+ * chunk_size_intra / chunk_size_inter (mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:28-31,118-121):
+ * chunk_size_inter is fixed at 128 here and state_stride = chunk_size_intra / 128.  0 = the default for the shape,
+ * otherwise 1 .. 8.  Results agree for every value within the rounding of bf16 operands.
+ *
+ * The forward (with keep_for_backward), both workspace queries and the backward of one pass must be called with the
+ * same path and state_stride: they decide the layout of the workspaces.
  */
 #define MLSTM_PATH_AUTO 0
 #define MLSTM_PATH_SPLIT 1
 #define MLSTM_PATH_FUSED 2
-int mlstm_hip_set_chunkwise_path(int path);
 
 /*
  * Fused recurrent decode step (one token for every (b, head)).
@@ -82,7 +91,8 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
  * workspace additionally holds everything the backward re-uses (gate vectors, per-chunk bf16 states,
  * per-row normalisers) and must be handed unchanged to mlstm_hip_chunkwise_bw.
  */
-size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int keep_for_backward);
+size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int keep_for_backward,
+                                              int path, int state_stride);
 
 /*
  * TFLA chunkwise forward, mLSTMexp or mLSTMsig.
@@ -99,10 +109,11 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
                            float* c_last, float* n_last, float* m_last,
                            void* workspace, size_t workspace_bytes, int keep_for_backward,
                            int B, int NH, int S, int DHQK, int DHHV, float eps,
-                           int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream);
+                           int dtype_qkv, int dtype_gates, int gate, int normalize, int path, int state_stride,
+                           void* stream);
 
 /* Bytes of scratch the chunkwise backward needs in addition to the forward workspace. */
-size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV);
+size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int state_stride);
 
 /*
  * TFLA chunkwise backward (normaliser and stabilisers are constants, as in the reference).
@@ -119,7 +130,8 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
                            const void* fw_workspace, size_t fw_workspace_bytes,
                            void* bw_workspace, size_t bw_workspace_bytes,
                            int B, int NH, int S, int DHQK, int DHHV, float eps,
-                           int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream);
+                           int dtype_qkv, int dtype_gates, int gate, int normalize, int path, int state_stride,
+                           void* stream);
 
 #ifdef __cplusplus
 }

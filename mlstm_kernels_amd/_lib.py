@@ -12,7 +12,7 @@ _lib = None
 F32, BF16 = 0, 1
 GATE_EXP, GATE_SIG = 0, 1
 PATH_AUTO, PATH_SPLIT, PATH_FUSED = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
 
@@ -20,13 +20,12 @@ _SIGNATURES = {
     "mlstm_hip_abi_version": (_i, []),
     "mlstm_hip_last_error": (ctypes.c_char_p, []),
     "mlstm_hip_profile_enable": (_i, [_i]),
-    "mlstm_hip_set_chunkwise_path": (_i, [_i]),
     "mlstm_hip_profile_read": (_i, [_i, ctypes.c_char_p, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)]),
     "mlstm_hip_step": (_i, [_vp] * 12 + [_i, _i, _i, _i, _f, _i, _i, _vp]),
-    "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 6),
-    "mlstm_hip_chunkwise_fw": (_i, [_vp] * 15 + [_sz, _i] + [_i] * 5 + [_f] + [_i] * 4 + [_vp]),
-    "mlstm_hip_chunkwise_bw_workspace_bytes": (_sz, [_i] * 5),
-    "mlstm_hip_chunkwise_bw": (_i, [_vp] * 14 + [_sz, _vp, _sz] + [_i] * 5 + [_f] + [_i] * 4 + [_vp]),
+    "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 8),
+    "mlstm_hip_chunkwise_fw": (_i, [_vp] * 15 + [_sz, _i] + [_i] * 5 + [_f] + [_i] * 6 + [_vp]),
+    "mlstm_hip_chunkwise_bw_workspace_bytes": (_sz, [_i] * 6),
+    "mlstm_hip_chunkwise_bw": (_i, [_vp] * 14 + [_sz, _vp, _sz] + [_i] * 5 + [_f] + [_i] * 6 + [_vp]),
 }
 
 
@@ -63,9 +62,15 @@ def get_lib() -> ctypes.CDLL:
     return _lib
 
 
-def set_chunkwise_path(path: int) -> int:
-    """Select the kernels of the chunkwise passes (PATH_AUTO / PATH_SPLIT / PATH_FUSED); returns the previous setting."""
-    return get_lib().mlstm_hip_set_chunkwise_path(int(path))
+_PATH_CODES = {"auto": PATH_AUTO, "split": PATH_SPLIT, "fused": PATH_FUSED}
+
+
+def path_code(name: str) -> int:
+    """'auto' / 'split' / 'fused' -> the C ABI's kernel path code."""
+    try:
+        return _PATH_CODES[name]
+    except KeyError:
+        raise ValueError(f"unknown kernel path {name!r}; expected one of {sorted(_PATH_CODES)}") from None
 
 
 def profile_enable(on: bool) -> None:

@@ -1,5 +1,6 @@
 // C ABI of libmlstm_hip.so (declared in include/mlstm_hip.h): argument validation, workspace carving and
-// kernel sequencing.  No device memory is allocated here and no state is kept between calls.
+// kernel sequencing.  No device memory is allocated here and no state is kept between calls (kernel path and state
+// stride are per-call arguments).
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -58,28 +59,40 @@ int check_launch(const char* what) {
 // Which kernels carry the value-column side of the chunkwise passes (H forward, dV backward):
 //   split : state scan, then a chunk-parallel kernel reading the materialised chunk states
 //   fused : one sequential kernel per pass that keeps the state slice in registers
-// The fused kernels move far fewer bytes (no chunk state is written or re-read by them) but run one workgroup per
-// (batch, head, 64 value columns) and per CU.
-int g_chunkwise_path = MLSTM_PATH_AUTO;
-bool use_fused(int B, int NH, int DHQK, int DHHV) {
-  if (g_chunkwise_path == MLSTM_PATH_SPLIT || !mlstm::fused_hv_supported(DHQK, DHHV)) return false;
-  // Measured on MI355X at B*S = 65536, NH = 8, 256/512: fused forward 1.56 ms against 1.48 ms split, fused dV 1.28 ms
-  // against 1.34 ms split.  With one four-wave workgroup per CU the fused kernels are latency-bound, so they are
-  // opt-in only.
-  (void)B; (void)NH;
-  return g_chunkwise_path == MLSTM_PATH_FUSED;
+// The fused kernels move far fewer bytes (no chunk state is written or re-read by them) but run one four-wave
+// workgroup per (batch, head, 64 value columns) and per CU, which leaves them latency-bound: measured on MI355X at
+// B*S = 65536, NH = 8, 256/512 the fused forward takes 1.56 ms against 1.08 ms split.  They are opt-in only.
+bool use_fused(int path, int DHQK, int DHHV) { return path == MLSTM_PATH_FUSED && mlstm::fused_hv_supported(DHQK, DHHV); }
+// Chunk states are kept every `stride` chunks of 128 positions (0 = the default for the shape).  Fewer kept states
+// mean less HBM traffic (a state is DHQK x DHHV bf16 per chunk and head, written once and read by three kernels)
+// against more score blocks in the chunk-parallel kernels.
+constexpr int kDefaultStateStride = 2;
+int resolve_stride(int state_stride) { return state_stride == 0 ? kDefaultStateStride : state_stride; }
+const char* check_options(int path, int state_stride, int DHQK, int DHHV) {
+  if (path != MLSTM_PATH_AUTO && path != MLSTM_PATH_SPLIT && path != MLSTM_PATH_FUSED) return "unknown kernel path code";
+  if (path == MLSTM_PATH_FUSED && !mlstm::fused_hv_supported(DHQK, DHHV))
+    return "the fused kernel path supports DHQK = 128 or 256 only";
+  if (state_stride < 0 || state_stride > mlstm::kMaxStateStride) return "state_stride must be 0 (default) or 1 .. 8";
+  return nullptr;
 }
 const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {
   if (B <= 0 || NH <= 0 || S <= 0) return "B, NH and S must be positive";
   if (DHQK <= 0 || DHHV <= 0 || DHQK % 64 != 0 || DHHV % 64 != 0) return "DHQK and DHHV must be positive multiples of 64";
   if ((long long)B * NH > 65535) return "B*NH exceeds 65535";
+  // the chunk-parallel kernels keep 64 rows of q or k resident in LDS (132 bytes per head-dimension entry beside
+  // 40 KB of tiles, 160 KB per workgroup at most)
+  if (DHQK > 896) return "DHQK too large for the LDS-resident tile (at most 896)";
   return nullptr;
 }
 }  // namespace
 
+namespace mlstm {
+int set_last_error(const char* msg) { return fail(msg); }
+}  // namespace mlstm
+
 extern "C" {
 
-int mlstm_hip_abi_version(void) { return 1; }
+int mlstm_hip_abi_version(void) { return 2; }
 
 int mlstm_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
@@ -119,12 +132,6 @@ int mlstm_hip_profile_read(int index, char* name, size_t name_cap, float* total_
 }
 const char* mlstm_hip_last_error(void) { return g_err; }
 
-int mlstm_hip_set_chunkwise_path(int path) {
-  const int previous = g_chunkwise_path;
-  if (path == MLSTM_PATH_AUTO || path == MLSTM_PATH_SPLIT || path == MLSTM_PATH_FUSED) g_chunkwise_path = path;
-  return previous;
-}
-
 int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c_in,
                    const float* n_in, const float* m_in, void* h, float* c_out, float* n_out, float* m_out, int B,
                    int NH, int DHQK, int DHHV, float eps, int dtype_qkv, int dtype_gates, void* stream) {
@@ -143,31 +150,41 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
   return check_launch("mlstm_hip_step");
 }
 
-size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int keep_for_backward) {
-  if (check_dims(B, NH, S, DHQK, DHHV)) return 0;
-  const bool with_states = keep_for_backward || !use_fused(B, NH, DHQK, DHHV);
-  return mlstm::carve_fw_workspace(nullptr, B, NH, S, DHQK, DHHV, with_states).bytes;
+size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int keep_for_backward, int path,
+                                              int state_stride) {
+  if (check_dims(B, NH, S, DHQK, DHHV) || check_options(path, state_stride, DHQK, DHHV)) return 0;
+  const bool with_states = keep_for_backward || !use_fused(path, DHQK, DHHV);
+  return mlstm::carve_fw_workspace(nullptr, B, NH, S, DHQK, DHHV, with_states, resolve_stride(state_stride)).bytes;
 }
 
-int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c0,
-                           const float* n0, const float* m0, void* H, float* n_out, float* m_out, float* c_last,
-                           float* n_last, float* m_last, void* workspace, size_t workspace_bytes,
-                           int keep_for_backward, int B, int NH, int S, int DHQK, int DHHV, float eps, int dtype_qkv,
-                           int dtype_gates, int gate, int normalize, void* stream) {
-  if (!q || !k || !v || !i || !f || !H || !workspace) return fail("mlstm_hip_chunkwise_fw: null pointer argument");
-  if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return fail(e);
-  if (dtype_qkv != MLSTM_BF16) return fail("mlstm_hip_chunkwise_fw: q/k/v must be bf16");
-  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return fail("mlstm_hip_chunkwise_fw: unsupported gate dtype");
-  if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return fail("mlstm_hip_chunkwise_fw: unknown gate code");
+}  // extern "C"
+
+namespace {
+// The forward pass proper: arguments validated, workspace carved from `workspace`.
+int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void* v, const void* i, const void* f,
+                      const float* c0, const float* n0, const float* m0, void* H, float* n_out, float* m_out,
+                      float* c_last, float* n_last, float* m_last, void* workspace, size_t workspace_bytes,
+                      int keep_for_backward, int B, int NH, int S, int DHQK, int DHHV, float eps, int dtype_qkv,
+                      int dtype_gates, int gate, int normalize, int path, int state_stride, hipStream_t st) {
+  char msg[160];
+  auto failw = [&](const char* what) {
+    snprintf(msg, sizeof(msg), "%s: %s", who, what);
+    return fail(msg);
+  };
+  if (!q || !k || !v || !i || !f || !H || !workspace) return failw("null pointer argument");
+  if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return failw(e);
+  if (const char* e = check_options(path, state_stride, DHQK, DHHV)) return failw(e);
+  if (dtype_qkv != MLSTM_BF16) return failw("q/k/v must be bf16");
+  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return failw("unsupported gate dtype");
+  if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return failw("unknown gate code");
   const bool has_c0 = c0 != nullptr;
-  if (has_c0 != (n0 != nullptr)) return fail("mlstm_hip_chunkwise_fw: c0 and n0 must be given together");
-  if (gate == MLSTM_GATE_EXP && has_c0 != (m0 != nullptr))
-    return fail("mlstm_hip_chunkwise_fw: initial states must be given together");
-  const bool fused = use_fused(B, NH, DHQK, DHHV);
+  if (has_c0 != (n0 != nullptr)) return failw("c0 and n0 must be given together");
+  if (gate == MLSTM_GATE_EXP && has_c0 != (m0 != nullptr)) return failw("initial states must be given together");
+  const bool fused = use_fused(path, DHQK, DHHV);
   const bool with_states = keep_for_backward || !fused;
-  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(workspace, B, NH, S, DHQK, DHHV, with_states);
-  if (workspace_bytes < ws.bytes) return fail("mlstm_hip_chunkwise_fw: workspace too small");
-  hipStream_t st = (hipStream_t)stream;
+  const int stride = resolve_stride(state_stride);
+  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(workspace, B, NH, S, DHQK, DHHV, with_states, stride);
+  if (workspace_bytes < ws.bytes) return failw("workspace too small");
   const int NC = (S + 127) / 128, BH = B * NH;
   const int sig = gate == MLSTM_GATE_SIG;
   {
@@ -180,7 +197,7 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   if (!track_n && n_last != nullptr) {
     if (n0 != nullptr) {
       if (hipMemcpyAsync(n_last, n0, (size_t)BH * DHQK * sizeof(float), hipMemcpyDeviceToDevice, st) != hipSuccess)
-        return fail("mlstm_hip_chunkwise_fw: copying n0 to n_last failed");
+        return failw("copying n0 to n_last failed");
     } else if (const char* e = mlstm::launch_fill_zero(n_last, (size_t)BH * DHQK, st)) {
       return fail(e);
     }
@@ -203,6 +220,7 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
     fa.eps = eps;
     fa.sig_gate = sig;
     fa.use_nrow = track_n;
+    fa.stride = stride;
     {
       ProfileScope ps("fused_fw", st);
       if (const char* e = mlstm::launch_fused_hv(fa, BH, /*is_dv=*/false, st)) return fail(e);
@@ -226,6 +244,7 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   sa.qk_scale = 1.0f / sqrtf((float)DHQK);
   sa.eps = eps;
   sa.backward = 0;
+  sa.stride = stride;
   {
     ProfileScope ps("scan_fw", st);
     if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/true, st)) return fail(e);
@@ -245,6 +264,7 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   pa.qk_scale = sa.qk_scale; pa.eps = eps;
   pa.sig_gate = sig;
   pa.use_nrow = !(sig && !normalize);
+  pa.stride = stride;
   {
     ProfileScope ps("par_h", st);
     if (const char* e = mlstm::launch_par_hv(pa, BH, /*is_dv=*/false, st)) return fail(e);
@@ -252,25 +272,44 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
   return check_launch("par_hv forward");
 }
 
-size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV) {
-  if (check_dims(B, NH, S, DHQK, DHHV)) return 0;
-  return mlstm::carve_bw_workspace(nullptr, B, NH, S, DHQK, DHHV).bytes;
+}  // namespace
+
+extern "C" {
+
+int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c0,
+                           const float* n0, const float* m0, void* H, float* n_out, float* m_out, float* c_last,
+                           float* n_last, float* m_last, void* workspace, size_t workspace_bytes,
+                           int keep_for_backward, int B, int NH, int S, int DHQK, int DHHV, float eps, int dtype_qkv,
+                           int dtype_gates, int gate, int normalize, int path, int state_stride, void* stream) {
+  return chunkwise_fw_impl("mlstm_hip_chunkwise_fw", q, k, v, i, f, c0, n0, m0, H, n_out, m_out, c_last, n_last, m_last,
+                           workspace, workspace_bytes, keep_for_backward, B, NH, S, DHQK, DHHV, eps, dtype_qkv,
+                           dtype_gates, gate, normalize, path, state_stride, (hipStream_t)stream);
+}
+
+size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int state_stride) {
+  if (check_dims(B, NH, S, DHQK, DHHV) || check_options(MLSTM_PATH_AUTO, state_stride, DHQK, DHHV)) return 0;
+  return mlstm::carve_bw_workspace(nullptr, B, NH, S, DHQK, DHHV, resolve_stride(state_stride),
+                                   DHQK / mlstm::par_qk_head_tile(DHQK)).bytes;
 }
 
 int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const void* i, const void* f, const void* dH,
                            const float* dC_last, void* dQ, void* dK, void* dV, float* dI, float* dF, float* dC0,
                            const void* fw_workspace, size_t fw_workspace_bytes, void* bw_workspace,
                            size_t bw_workspace_bytes, int B, int NH, int S, int DHQK, int DHHV, float eps,
-                           int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream) {
+                           int dtype_qkv, int dtype_gates, int gate, int normalize, int path, int state_stride,
+                           void* stream) {
   if (!q || !k || !v || !i || !f || !dH || !dQ || !dK || !dV || !dI || !dF || !fw_workspace || !bw_workspace)
     return fail("mlstm_hip_chunkwise_bw: null pointer argument");
   if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return fail(e);
+  if (const char* e = check_options(path, state_stride, DHQK, DHHV)) return fail(e);
   if (dtype_qkv != MLSTM_BF16) return fail("mlstm_hip_chunkwise_bw: q/k/v/dH must be bf16");
   if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return fail("mlstm_hip_chunkwise_bw: unsupported gate dtype");
   if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return fail("mlstm_hip_chunkwise_bw: unknown gate code");
-  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(const_cast<void*>(fw_workspace), B, NH, S, DHQK, DHHV, true);
+  const int stride = resolve_stride(state_stride);
+  const int tiles = DHQK / mlstm::par_qk_head_tile(DHQK);
+  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(const_cast<void*>(fw_workspace), B, NH, S, DHQK, DHHV, true, stride);
   if (fw_workspace_bytes < ws.bytes) return fail("mlstm_hip_chunkwise_bw: forward workspace too small");
-  mlstm::BwWorkspace bws = mlstm::carve_bw_workspace(bw_workspace, B, NH, S, DHQK, DHHV);
+  mlstm::BwWorkspace bws = mlstm::carve_bw_workspace(bw_workspace, B, NH, S, DHQK, DHHV, stride, tiles);
   if (bw_workspace_bytes < bws.bytes) return fail("mlstm_hip_chunkwise_bw: backward workspace too small");
   hipStream_t st = (hipStream_t)stream;
   const int NC = (S + 127) / 128, BH = B * NH;
@@ -278,7 +317,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   const int use_nrow = !(sig && !normalize);
   const float qk_scale = 1.0f / sqrtf((float)DHQK);
 
-  if (use_fused(B, NH, DHQK, DHHV)) {
+  if (use_fused(path, DHQK, DHHV)) {
     mlstm::FusedHvArgs fa;
     memset(&fa, 0, sizeof(fa));
     fa.Q = (const uint16_t*)q; fa.K = (const uint16_t*)k; fa.V = (const uint16_t*)v; fa.dH = (const uint16_t*)dH;
@@ -291,54 +330,51 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
     fa.S = S; fa.NC = NC; fa.DHQK = DHQK; fa.DHHV = DHHV;
     fa.qk_scale = qk_scale; fa.eps = eps;
     fa.sig_gate = sig; fa.use_nrow = use_nrow;
+    fa.stride = stride;
     {
       ProfileScope ps("fused_dv", st);
       if (const char* e = mlstm::launch_fused_hv(fa, BH, /*is_dv=*/true, st)) return fail(e);
     }
     if (check_launch("fused_hv dV")) return 1;
   } else {
-  mlstm::ScanArgs sa;
-  memset(&sa, 0, sizeof(sa));
-  sa.X = (const uint16_t*)q;
-  sa.Y = (const uint16_t*)dH;
-  sa.scale_a = ws.g.bbar;
-  sa.nrow = use_nrow ? ws.nrow : nullptr;
-  sa.gbar = ws.g.gbar;
-  sa.init = dC_last;
-  sa.states = bws.dcstates;
-  sa.final_out = dC0;
-  sa.S = S; sa.NC = NC; sa.DHQK = DHQK; sa.DHHV = DHHV;
-  sa.qk_scale = qk_scale; sa.eps = eps;
-  sa.backward = 1;
-  {
-    ProfileScope ps("scan_bw", st);
-    if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/false, st)) return fail(e);
-  }
-  if (check_launch("scan_bw")) return 1;
+    mlstm::ScanArgs sa;
+    memset(&sa, 0, sizeof(sa));
+    sa.X = (const uint16_t*)q;
+    sa.Y = (const uint16_t*)dH;
+    sa.scale_a = ws.g.bbar;
+    sa.nrow = use_nrow ? ws.nrow : nullptr;
+    sa.gbar = ws.g.gbar;
+    sa.init = dC_last;
+    sa.states = bws.dcstates;
+    sa.final_out = dC0;
+    sa.S = S; sa.NC = NC; sa.DHQK = DHQK; sa.DHHV = DHHV;
+    sa.qk_scale = qk_scale; sa.eps = eps;
+    sa.backward = 1;
+    sa.stride = stride;
+    {
+      ProfileScope ps("scan_bw", st);
+      if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/false, st)) return fail(e);
+    }
+    if (check_launch("scan_bw")) return 1;
 
-  mlstm::ParHvArgs pv;
-  memset(&pv, 0, sizeof(pv));
-  pv.Q = (const uint16_t*)q; pv.K = (const uint16_t*)k; pv.V = (const uint16_t*)v; pv.dH = (const uint16_t*)dH;
-  pv.g = ws.g;
-  pv.states = bws.dcstates;
-  pv.nrow = ws.nrow;
-  pv.Out = (uint16_t*)dV;
-  pv.S = S; pv.NC = NC; pv.DHQK = DHQK; pv.DHHV = DHHV;
-  pv.qk_scale = qk_scale; pv.eps = eps;
-  pv.sig_gate = sig; pv.use_nrow = use_nrow;
-  {
-    ProfileScope ps("par_dv", st);
-    if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
-  }
-  if (check_launch("par_hv dV")) return 1;
+    mlstm::ParHvArgs pv;
+    memset(&pv, 0, sizeof(pv));
+    pv.Q = (const uint16_t*)q; pv.K = (const uint16_t*)k; pv.V = (const uint16_t*)v; pv.dH = (const uint16_t*)dH;
+    pv.g = ws.g;
+    pv.states = bws.dcstates;
+    pv.nrow = ws.nrow;
+    pv.Out = (uint16_t*)dV;
+    pv.S = S; pv.NC = NC; pv.DHQK = DHQK; pv.DHHV = DHHV;
+    pv.qk_scale = qk_scale; pv.eps = eps;
+    pv.sig_gate = sig; pv.use_nrow = use_nrow;
+    pv.stride = stride;
+    {
+      ProfileScope ps("par_dv", st);
+      if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
+    }
+    if (check_launch("par_hv dV")) return 1;
   }
 
-  const int MT = DHQK % 256 == 0 ? 256 : (DHQK % 128 == 0 ? 128 : 64);
-  if (DHQK / MT > 1) {
-    // several head-dim tiles accumulate their row dots atomically: start from zero (qdq and kdk are adjacent)
-    const size_t n = (size_t)((char*)bws.kdk - (char*)bws.qdq) / 4 + (size_t)BH * NC * 128;
-    if (const char* e = mlstm::launch_fill_zero(bws.qdq, n, st)) return fail(e);
-  }
   mlstm::ParQkArgs pq;
   memset(&pq, 0, sizeof(pq));
   pq.Q = (const uint16_t*)q; pq.K = (const uint16_t*)k; pq.V = (const uint16_t*)v; pq.dH = (const uint16_t*)dH;
@@ -347,6 +383,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   pq.S = S; pq.NC = NC; pq.DHQK = DHQK; pq.DHHV = DHHV;
   pq.qk_scale = qk_scale; pq.eps = eps;
   pq.use_nrow = use_nrow;
+  pq.stride = stride;
   // dQ and dK in one launch: the workgroups of a chunk run side by side and share the Q, K, V and dH rows they stream
   pq.states = ws.cstates; pq.Out = (uint16_t*)dQ; pq.rowdot = bws.qdq;
   pq.states2 = bws.dcstates; pq.Out2 = (uint16_t*)dK; pq.rowdot2 = bws.kdk;
@@ -359,6 +396,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   mlstm::GateGradArgs ga;
   memset(&ga, 0, sizeof(ga));
   ga.i = i; ga.f = f; ga.qdq = bws.qdq; ga.kdk = bws.kdk; ga.dI = dI; ga.dF = dF;
+  ga.ntiles = tiles;
   ga.S = S; ga.NC = NC; ga.dtype_gates = dtype_gates; ga.sig_gate = sig;
   {
     ProfileScope ps("gate_grads", st);

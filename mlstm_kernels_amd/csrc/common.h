@@ -64,6 +64,15 @@ __device__ __forceinline__ uint2 lds_read_tr16(const void* p) {
   return c.u;
 }
 
+// A copy of x the optimiser knows nothing about.  Index arithmetic derived from it inside a loop body is redone in
+// every iteration instead of being hoisted out of the loop into registers that stay live (and get spilled) for the
+// whole kernel; the handful of integer instructions per iteration is far cheaper than a spill reload, which queues
+// behind the global loads in flight.
+__device__ __forceinline__ int opaque(int x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
 __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);

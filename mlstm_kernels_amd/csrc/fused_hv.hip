@@ -246,12 +246,6 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
   const int n = 32 * nb + r;  // position inside the chunk of this lane's output row / score column
   constexpr float kLog2e = 1.4426950408889634f;
   const float log2_qk = __log2f(a.qk_scale);
-#ifdef MLSTM_FUSED_TIMING
-  unsigned long long tph[6] = {0, 0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
-#define MLSTM_TICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
-#else
-#define MLSTM_TICK(p_)
-#endif
   for (int it = 0; it < NC; ++it) {
     const int c = c_first + it * c_step;
     const int t_base = c * kChunk;
@@ -319,8 +313,13 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
       }
       // state before this chunk's update -> bf16 fragments: LDS (natural order of the contraction index, so that
       // Xn fragments are plain 16-byte loads of a row) and, on request, HBM (the stored fragment format)
-      u32x4* stg = a.states == nullptr ? nullptr
-                                       : (u32x4*)a.states + ((size_t)bh * NC + c) * (size_t)(DHHV / 32) * ND * 64;
+      // kept boundaries only: forward the state before every stride-th chunk, dV the gradient of the state after the
+      // last chunk of every group of `stride` chunks (and after the last chunk of the sequence); slot c / stride
+      const bool keep_state = IS_DV ? (c == NC - 1 || (c + 1) % a.stride == 0) : (c % a.stride == 0);
+      const size_t NCS = (size_t)(NC + a.stride - 1) / a.stride;
+      u32x4* stg = (a.states == nullptr || !keep_state)
+                       ? nullptr
+                       : (u32x4*)a.states + ((size_t)bh * NCS + c / a.stride) * (size_t)(DHHV / 32) * ND * 64;
 #pragma unroll
       for (int db = 0; db < DBW; ++db)
 #pragma unroll
@@ -340,9 +339,7 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
             if (stg != nullptr) stg[((size_t)((w_tile >> 5) + wb) * ND + D16) * 64 + lane] = f;
           }
     }
-    MLSTM_TICK(0)
     __syncthreads();  // ---- everything staged for this chunk is visible; from here on the waves run independently
-    MLSTM_TICK(5)
     const float gdec = gdl[it & 1];  // decay of this chunk (through LDS: no dependence on loads in flight)
 
     // =========================== inter-chunk product ===========================
@@ -383,7 +380,6 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
     const float csn = cs[n];
 #pragma unroll
     for (int wb = 0; wb < WPW; ++wb) oacc[wb] *= csn;
-    MLSTM_TICK(1)
 
     // =========================== score blocks, gated in registers, times the value rows ===========================
     // A gated 32x32 score block never leaves the wave: in accumulator layout lane (r, h) holds, for its column n,
@@ -488,7 +484,6 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
         }
       }
     }
-    MLSTM_TICK(2)
 
     // =========================== state update ===========================
 #pragma unroll
@@ -526,7 +521,6 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
         if (d < DQ) nvn[d] = gdec * nvc[d] + nsum[k];
       }
     }
-    MLSTM_TICK(3)
 
     // =========================== output rows ===========================
     {
@@ -546,15 +540,8 @@ __global__ __launch_bounds__(256 * NWQ) __attribute__((amdgpu_waves_per_eu(NWQ, 
       MLSTM_LOAD_XN(c + c_step);
       MLSTM_PUBLISH_SCALE((it + 1) & 1, c + c_step);
     }
-    MLSTM_TICK(4)
     __syncthreads();  // ---- every wave is done with this chunk's tiles
-    MLSTM_TICK(5)
   }
-#ifdef MLSTM_FUSED_TIMING
-  if (blockIdx.x == 0 && blockIdx.y == 0 && lane == 0)
-    for (int p = 0; p < 6; ++p) a.timing[(wave & 7) * 8 + p] = tph[p];
-#endif
-#undef MLSTM_TICK
 #undef MLSTM_PREFETCH_KV
 #undef MLSTM_PREFETCH_GATES
 #undef MLSTM_LOAD_XN
@@ -595,9 +582,10 @@ bool fused_hv_supported(int DHQK, int DHHV) { return (DHQK == 128 || DHQK == 256
 
 const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
   if (!fused_hv_supported(a.DHQK, a.DHHV)) return "fused_hv: unsupported head dimensions";
-#ifndef MLSTM_FUSED_NWQ
-#define MLSTM_FUSED_NWQ 1
-#endif
+  if (a.stride < 1 || a.stride > kMaxStateStride) return "fused_hv: state stride out of range";
+  // one wave per 32-position block (four waves, one per SIMD): the eight-wave form, in which the two waves of a block
+  // both compute its scores, was measured slower
+  constexpr int MLSTM_FUSED_NWQ = 1;
   if (is_dv) {
     if (a.DHQK == 256) return launch_fused_hv_t<256, true, false, MLSTM_FUSED_NWQ>(a, BH, stream);
     return launch_fused_hv_t<128, true, false, MLSTM_FUSED_NWQ>(a, BH, stream);

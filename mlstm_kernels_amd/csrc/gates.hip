@@ -219,11 +219,22 @@ __global__ __launch_bounds__(kGateThreads) void gate_grads_kernel(GateGradArgs a
   const size_t Sp = (size_t)a.NC * kChunk;
   const float* qdq = a.qdq + bh * Sp;
   const float* kdk = a.kdk + bh * Sp;
+  const size_t tile_stride = (size_t)gridDim.y * Sp;  // the row dots come in one slot per head-dimension tile
+  auto diff = [&](int t) {  // q.dQ - k.dK of position t, tiles summed in a fixed order
+    float s = 0.f;
+    for (int tl = 0; tl < a.ntiles; ++tl) s += qdq[tl * tile_stride + t] - kdk[tl * tile_stride + t];
+    return s;
+  };
+  auto kdot = [&](int t) {
+    float s = 0.f;
+    for (int tl = 0; tl < a.ntiles; ++tl) s += kdk[tl * tile_stride + t];
+    return s;
+  };
   const int seg_lo = blockIdx.x * kGradSeg;
   const int seg_hi = min(seg_lo + kGradSeg, S);
   // everything behind this segment
   float part = 0.f;
-  for (int t = seg_hi + tid; t < S; t += kGateThreads) part += qdq[t] - kdk[t];
+  for (int t = seg_hi + tid; t < S; t += kGateThreads) part += diff(t);
   part = wave_sum(part);
   if (lane == 0) wtot[wave] = part;
   __syncthreads();
@@ -236,8 +247,8 @@ __global__ __launch_bounds__(kGateThreads) void gate_grads_kernel(GateGradArgs a
   float kd[2], d[2];
 #pragma unroll
   for (int e = 0; e < 2; ++e) {
-    kd[e] = t0 + e < S ? kdk[t0 + e] : 0.f;
-    d[e] = t0 + e < S ? qdq[t0 + e] - kd[e] : 0.f;
+    kd[e] = t0 + e < S ? kdot(t0 + e) : 0.f;
+    d[e] = t0 + e < S ? diff(t0 + e) : 0.f;
   }
   const float pair = d[0] + d[1];
   auto add = [](float x, float y) { return x + y; };
@@ -266,6 +277,7 @@ __global__ void fill_zero_kernel(float* p, size_t n) {
 }
 
 const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream) {
+  if (a.ntiles < 1) return "gate_grads: the row dots need at least one tile slot";
   hipLaunchKernelGGL(gate_grads_kernel, dim3((a.S + kGradSeg - 1) / kGradSeg, BH), dim3(kGateThreads), 0, stream, a);
   return nullptr;
 }

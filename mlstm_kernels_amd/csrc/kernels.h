@@ -16,7 +16,7 @@ struct ScanArgs {
   const float* nrow;      // backward: [BH][Sp] row normaliser or nullptr; forward: nullptr
   const float* gbar;      // [BH][NC]
   const float* init;      // (B,NH,DHQK,DHHV) fp32 or nullptr (zeros)
-  uint16_t* states;       // bf16 fragments [BH][NC][DHHV/32][DHQK/16][64][8]
+  uint16_t* states;       // bf16 fragments [BH][ceil(NC/stride)][DHHV/32][DHQK/16][64][8]
   float* final_out;       // (B,NH,DHQK,DHHV) fp32 or nullptr
   const float* n_init;    // forward: (B,NH,DHQK) or nullptr
   float* nstates;         // forward: [BH][NC][DHQK] or nullptr (skip the n recurrence)
@@ -24,9 +24,7 @@ struct ScanArgs {
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
   int backward;
-#ifdef MLSTM_SCAN_TIMING
-  unsigned long long* timing;  // one-off timing builds
-#endif
+  int stride;             // a chunk state is kept every `stride` chunks
 };
 
 struct ParHvArgs {
@@ -43,9 +41,7 @@ struct ParHvArgs {
   float qk_scale, eps;
   int sig_gate;
   int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant
-#ifdef MLSTM_PAR_TIMING
-  unsigned long long* timing;  // one-off timing builds: per-wave cycle counts of the phases of one chunk's workgroups
-#endif
+  int stride;               // a chunk state is kept every `stride` chunks
 };
 
 struct FusedHvArgs {
@@ -54,7 +50,7 @@ struct FusedHvArgs {
   const float* init;        // (B,NH,DHQK,DHHV) fp32 initial state (forward: C0, dV: dC_last) or nullptr (zeros)
   const float* n_init;      // forward: (B,NH,DHQK) or nullptr
   const float* nrow;        // dV: row normaliser of the forward pass
-  uint16_t* states;         // bf16 state fragments [BH][NC][DHHV/32][DHQK/16][64][8] or nullptr (not emitted)
+  uint16_t* states;         // bf16 state fragments [BH][ceil(NC/stride)][DHHV/32][DHQK/16][64][8] or nullptr (not emitted)
   uint16_t* Out;            // (B,NH,S,DHHV) bf16: H or dV
   float* nrow_out;          // forward: row normaliser (workspace [BH][Sp])
   float* n_out;             // forward, optional (B,NH,S)
@@ -65,9 +61,7 @@ struct FusedHvArgs {
   float qk_scale, eps;
   int sig_gate;
   int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant (n is then not tracked)
-#ifdef MLSTM_FUSED_TIMING
-  unsigned long long* timing;  // one-off timing builds: per-wave cycle counts of the phases of workgroup (0,0)
-#endif
+  int stride;               // a chunk state is emitted every `stride` chunks
 };
 
 struct ParQkArgs {
@@ -76,21 +70,20 @@ struct ParQkArgs {
   const uint16_t* states;   // dQ: C states; dK: dC states
   const float* nrow;
   uint16_t* Out;            // (B,NH,S,DHQK) bf16: dQ or dK
-  float* rowdot;            // [BH][Sp]: sum_d q*dQ (dQ) or sum_d k*dK (dK)
+  float* rowdot;            // [DHQK tiles][BH][Sp]: sum_d q*dQ (dQ) or sum_d k*dK (dK) over the rows of one tile
   const uint16_t* states2;  // the dK operands (dC states, dK, sum_d k*dK); states, Out and rowdot above are the
   uint16_t* Out2;           // dQ operands
   float* rowdot2;
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
   int use_nrow;
-#ifdef MLSTM_PAR_TIMING
-  unsigned long long* timing;  // one-off timing builds
-#endif
+  int stride;               // a chunk state is kept every `stride` chunks
 };
 
 struct GateGradArgs {
   const void *i, *f;        // gate pre-activations (B,NH,S)
-  const float *qdq, *kdk;   // [BH][Sp]
+  const float *qdq, *kdk;   // [ntiles][BH][Sp]: one slot per head-dimension tile of the dQ/dK kernel
+  int ntiles;
   float *dI, *dF;           // (B,NH,S) fp32
   int S, NC, dtype_gates, sig_gate;
 };
@@ -106,7 +99,10 @@ const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t st
 bool fused_hv_supported(int DHQK, int DHHV);
 const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 const char* launch_par_qk_pair(const ParQkArgs& a, int BH, hipStream_t stream);
+int par_qk_head_tile(int DHQK);  // head-dimension rows per workgroup of the dQ/dK kernel
 const char* launch_gate_grads(const GateGradArgs& a, int BH, hipStream_t stream);
 const char* launch_fill_zero(float* p, size_t n, hipStream_t stream);
+// stores `msg` as the calling thread's last error (what mlstm_hip_last_error returns) and returns 1
+int set_last_error(const char* msg);
 
 }  // namespace mlstm

@@ -6,7 +6,8 @@
 //   stabiliser     mstates                     fp32 [B*NH][NC+1]   (index c = value before chunk c)
 //   normaliser     nstates                     fp32 [B*NH][NC][DHQK] (n before chunk c)
 //   row normaliser nrow                        fp32 [B*NH][NC*128]  max(|den|, floor), without eps
-//   chunk states   cstates                     bf16 [B*NH][NC][DHHV/32][DHQK/16][64 lanes][8]
+//   chunk states   cstates                     bf16 [B*NH][ceil(NC/stride)][DHHV/32][DHQK/16][64 lanes][8]
+//                  (the state before every stride-th chunk; stride 1 keeps all of them)
 //
 // A chunk state is stored as ready-made MFMA operand fragments of C^T: fragment (wb, ds) holds, for lane
 // l = 32*h + r and element e, the value C[16*ds + 8*(e/4) + 4*h + e%4][32*wb + r].  That is exactly how the
@@ -19,6 +20,8 @@
 #include <stdint.h>
 
 namespace mlstm {
+
+constexpr int kMaxStateStride = 8;  // chunk states are kept every 1 .. 8 chunks
 
 struct GateBufs {
   float *u, *w, *abar, *bbar, *mcomb, *gbar, *amax, *mstates;
@@ -34,17 +37,19 @@ struct FwWorkspace {
 };
 
 struct BwWorkspace {
-  uint16_t* dcstates;  // same fragment layout as cstates; index c = gradient of the state after chunk c
-  float* qdq;          // fp32 [B*NH][NC*128]: sum_d q*dQ per position
-  float* kdk;          // fp32 [B*NH][NC*128]: sum_d k*dK per position
+  uint16_t* dcstates;  // same fragment layout as cstates; slot s = gradient of the state after the last chunk of group s
+  float* qdq;          // fp32 [tiles][B*NH][NC*128]: sum_d q*dQ per position and head-dimension tile
+  float* kdk;          // fp32 [tiles][B*NH][NC*128]: sum_d k*dK per position and head-dimension tile
   size_t bytes;
 };
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // with_states = false leaves out the chunk states (forward passes whose states nobody reads: cstates is null)
-inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK, int DHHV, bool with_states) {
+inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK, int DHHV, bool with_states,
+                                      int stride) {
   const size_t BH = (size_t)B * NH, NC = (size_t)(S + 127) / 128, Sp = NC * 128;
+  const size_t NCS = (NC + stride - 1) / stride;
   char* p = (char*)base;
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -64,13 +69,14 @@ inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK
   w.g.graw = (float*)take(BH * NC * 4);
   w.nstates = (float*)take(BH * NC * DHQK * 4);
   w.nrow = (float*)take(BH * Sp * 4);
-  w.cstates = with_states ? (uint16_t*)take(BH * NC * (size_t)DHQK * DHHV * 2) : nullptr;
+  w.cstates = with_states ? (uint16_t*)take(BH * NCS * (size_t)DHQK * DHHV * 2) : nullptr;
   w.bytes = off;
   return w;
 }
 
-inline BwWorkspace carve_bw_workspace(void* base, int B, int NH, int S, int DHQK, int DHHV) {
+inline BwWorkspace carve_bw_workspace(void* base, int B, int NH, int S, int DHQK, int DHHV, int stride, int tiles) {
   const size_t BH = (size_t)B * NH, NC = (size_t)(S + 127) / 128, Sp = NC * 128;
+  const size_t NCS = (NC + stride - 1) / stride;
   char* p = (char*)base;
   size_t off = 0;
   auto take = [&](size_t bytes) {
@@ -79,9 +85,9 @@ inline BwWorkspace carve_bw_workspace(void* base, int B, int NH, int S, int DHQK
     return r;
   };
   BwWorkspace w;
-  w.dcstates = (uint16_t*)take(BH * NC * (size_t)DHQK * DHHV * 2);
-  w.qdq = (float*)take(BH * Sp * 4);
-  w.kdk = (float*)take(BH * Sp * 4);
+  w.dcstates = (uint16_t*)take(BH * NCS * (size_t)DHQK * DHHV * 2);
+  w.qdq = (float*)take((size_t)tiles * BH * Sp * 4);
+  w.kdk = (float*)take((size_t)tiles * BH * Sp * 4);
   w.bytes = off;
   return w;
 }

@@ -7,48 +7,53 @@
 // backward dV (mlstm_kernels/torch/chunkwise/native/bw.py:153-198), per chunk:
 //   dV[j][:]   = sum_t Sbar[t][j] rho_t dH[t][:]  +  abar_j * k_j^T dC_next          rho_t = 1/(nrow_t + eps)
 //
+// Chunk states are kept only every `stride`-th chunk (the counterpart of the reference's chunk_size_inter <
+// chunk_size_intra with save_states_every_nth_chunk, mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:28-31,
+// 118-121).  A chunk c whose own boundary state was not kept uses the nearest kept one and adds the chunks in between
+// as further score blocks without a causal mask: with c0 the last kept boundary at or before c,
+//   H[t]  = bbar_t e^{G(c0,c) + m_{c0} - m_c}/sqrt(d) q_t^T C_{c0}  +  sum_{c'=c0}^{c} sum_{j in c'} Sbar'[t][j] v_j,
+//   Sbar'[t][j] = (q_t . k_j)/sqrt(d) exp(u_t - w_j + G(c',c)),   G(a,b) = sum_{x=a}^{b-1} (sum of logsig(f) over chunk x)
+// (u, w are the within-chunk gate vectors of the chunk t resp. j lives in; every exponent stays <= 0), and dV is the
+// mirror image with the nearest kept dC boundary at or after the chunk.  The denominators need no change: n is
+// kept for every chunk (it is a vector).
+//
 // Both are the same GEMM chain on a transposed output tile  Out^T[w][n]  (value columns x chunk positions):
-//   Out^T = ( State^T[w][d] . Xn^T[d][n] ) * colscale[n]  +  Xw^T[w][o] . P[o][n]
-// with  n = query position t, o = key position j, Xn = Q, Xw = V, State = C_prev       (forward)
-//       n = key position j,   o = query position t, Xn = K, Xw = dH, State = dC_next   (dV)
+//   Out^T = ( State^T[w][d] . Xn^T[d][n] ) * colscale[n]  +  sum over source chunks  Xw^T[w][o] . P[o][n]
+// with  n = query position t, o = key position j, Xn = Q, Xw = V, State = C       (forward)
+//       n = key position j,   o = query position t, Xn = K, Xw = dH, State = dC   (dV)
 //   * State^T arrives as ready-made bf16 MFMA fragments written by the scan kernel (16 B per lane, no LDS),
 //     prefetched several contraction steps ahead in registers,
-//   * the 64 rows of Xn this workgroup owns stay resident in LDS (they feed the score matrix, the inter-chunk
+//   * the 64 rows of Xn this workgroup owns stay resident in LDS (they feed the score blocks, the inter-chunk
 //     product and, forward, q.n),
 //   * colscale multiplies the fp32 accumulator after the inter-chunk product (positions are accumulator
 //     columns), so Xn is never rescaled or re-rounded,
-//   * the gated score matrix P is produced cooperatively (fp32 gating, bf16 into LDS); only the blocks on or
-//     below the causal diagonal are computed,
+//   * per source chunk the gated score block P (64 x 128) is produced cooperatively (fp32 gating, bf16 into LDS)
+//     and consumed at once by all value columns of the group: the accumulators of up to two column tiles are live
+//     together, so a score block is computed once and never kept,
 //   * Xw^T fragments come from row-major slabs through the transposing LDS read; every slab is fetched from
 //     global memory into registers while the previous one is being multiplied.
-// A workgroup owns 64 positions (half a chunk).  The resident rows, the gated score matrix and (forward) the
-// denominators are built once; then the workgroup walks the value dimension in tiles of WT columns, its WT/MW waves
-// splitting a tile.  The footprint (about 73 KB of LDS) lets two workgroups share a CU; at WT = 256, MW = 32 that is
-// sixteen waves per CU, four instruction streams per SIMD to overlap memory, LDS and matrix latencies.
-//
-// Measured on MI355X at B=4, S=16384, 256/512 and not kept: the whole tile's state fragments in flight (PD = 16: spills
-// at 128 registers, 0.74 ms against 0.62 ms); four waves of 64 columns (0.61 against 0.585 ms); launching the chunks
-// whose states the scan wrote last first, chunk-major (no change: the memory-side cache does not hold them).
+// A workgroup owns 64 positions (half a chunk) and walks the value dimension in groups of NTG tiles of WT columns, its
+// WT/MW waves splitting a tile.  The footprint (about 73 KB of LDS) lets two workgroups share a CU; at WT = 256,
+// MW = 32 that is sixteen waves per CU, four instruction streams per SIMD to overlap memory, LDS and matrix latencies.
 #include "common.h"
 #include "kernels.h"
 
 namespace mlstm {
 
-#ifndef MLSTM_PAR_HV_MW256
-#define MLSTM_PAR_HV_MW256 32
-#endif
-
 // PD = how many contraction steps ahead the state fragments are fetched (must divide DHQK / 16).
-// MW = value columns per wave (64 or 32): WT / MW waves share the tile.
+// MW = value columns per wave (64 or 32): WT / MW waves share a tile.  NTG = column tiles per group (1 or 2).
 #define PAR_HV_WPE(WT_, MW_) ((WT_) / (MW_) >= 8 ? 4 : ((WT_) >= 128 ? 2 : 1))
-template <int WT, bool IS_DV, int PD, int MW>
+template <int WT, int NTG, bool IS_DV, int PD, int MW>
 __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId blk) {
-  constexpr int NWAVE = WT / MW;   // each wave owns MW value columns = MB MFMA row blocks
+  constexpr int NWAVE = WT / MW;   // each wave owns MW value columns of every tile of the group = MB MFMA row blocks
   constexpr int MB = MW / 32;
   constexpr int NTH = 64 * NWAVE;
-  constexpr int PS = 128 + 8;      // score matrix row stride: P stored as Ps[n][o]
+  constexpr int GW = WT * NTG;     // value columns per group
+  constexpr int JL = GW > 256 ? 1 : 2;  // contraction steps (16 rows) per value slab
+  constexpr int VR = 16 * JL;      // rows per value slab
+  constexpr int PS = 128 + 8;      // score block row stride: P stored as Ps[n][o]
   constexpr int KS = 64 + 8;       // slab row stride of the streamed score operand
-  constexpr int VS = WT + 32;      // slab row stride of the streamed value-side operand (rows 64 bytes apart in the banks)
+  constexpr int VS = GW + 32;      // slab row stride of the streamed value-side operand (rows 64 bytes apart in the banks)
   constexpr int HS = WT + 8;       // output staging row stride
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   const int QS = DHQK + 8;
@@ -57,66 +62,84 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   uint16_t* Ns = (uint16_t*)smem_raw;  // resident Xn rows [64][DHQK] in fragment order
   uint16_t* Ps = Ns + n_region;
   uint16_t* Ts = Ps + 64 * PS;
-  constexpr int t_region = (128 * KS > 32 * VS) ? 128 * KS : 32 * VS;
-  float* uu = (float*)(Ts + t_region);  // [128] u_t of the chunk
-  float* ww = uu + 128;                 // [128] w_j of the chunk
-  float* cs = ww + 128;                 // [64] column scale of this workgroup's positions
-  float* inv = cs + 64;                 // forward: [64] 1/(nmax + eps); dV: [128] rho_t of the chunk
-  float* rows = inv + 128;              // [8][32] partial row sums of Sbar per score unit (forward)
+  constexpr int t_region = (128 * KS > VR * VS) ? 128 * KS : VR * VS;
+  static_assert(t_region >= 32 * HS, "the slab buffer also stages 32 output rows");
+  float* nvec = (float*)(Ts + t_region);  // [64] gate vector of this workgroup's positions: u_t (forward) / w_j (dV)
+  float* ovec = nvec + 64;              // [128] gate vector of the source chunk: w_j (forward) / u_t (dV)
+  float* orho = ovec + 128;             // [128] dV: rho_t of the source chunk
+  float* cs = orho + 128;               // [64] column scale of the inter-chunk product
+  float* inv = cs + 64;                 // [64] forward: 1/(nmax + eps)
+  float* rows = inv + 64;               // [8][32] partial row sums of Sbar per score unit (forward)
   float* nperm = rows + 8 * 32;         // [DHQK] n_prev in fragment order (forward)
   float* mcs = nperm + DHQK;            // [64] combined stabiliser of this workgroup's positions (forward)
+  float* cs0 = mcs + 64;                // [64] forward: bbar_t/sqrt(d), the weight of q.n_prev in the denominator
 
   // the wave index is made scalar so that branches on it are scalar branches (accumulators stay in place)
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-#ifdef MLSTM_PAR_TIMING
-  unsigned long long tph[7] = {0, 0, 0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
-#define MLSTM_PTICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
-#else
-#define MLSTM_PTICK(p_)
-#endif
   const int bh = blk.z, c = blk.y;
   const int nh = blk.x;                // which half of the chunk's positions
-  const int NWT = DHHV / WT;           // column tiles, handled one after the other by this workgroup
+  const int NG = DHHV / GW;            // column groups, handled one after the other by this workgroup
   const size_t Sp = (size_t)NC * kChunk;
-  const size_t gofs = bh * Sp + (size_t)c * kChunk;
+  const size_t hofs = bh * Sp;
+  const size_t gofs = hofs + (size_t)c * kChunk;
   const int t_base = c * kChunk;
   const int n0 = 64 * nh;              // first position (inside the chunk) of this workgroup
-  // live 32-row blocks of the other position index o: forward o = j <= t, dV o = t >= j
-  const int ob_lo = IS_DV ? 2 * nh : 0, ob_hi = IS_DV ? 4 : 2 * (nh + 1);
+  const int stride = a.stride;
+  const int slot = c / stride;         // kept boundary state this chunk uses
+  // source chunks of the score blocks: forward c0 .. c (own chunk last), dV c .. c1 (own chunk first)
+  const int sc_lo = IS_DV ? c : slot * stride;
+  const int sc_hi = IS_DV ? min(slot * stride + stride - 1, NC - 1) : c;
   const uint16_t* Xn_g = (IS_DV ? a.K : a.Q) + (size_t)bh * S * DHQK;
   const uint16_t* Xo_g = (IS_DV ? a.Q : a.K) + (size_t)bh * S * DHQK;
   const uint16_t* Xw_g = (IS_DV ? a.dH : a.V) + (size_t)bh * S * DHHV;
+  const float* graw = a.g.graw + (size_t)bh * NC;
+  const float* mst = a.g.mstates + (size_t)bh * (NC + 1);
+
+  // live 32-row blocks of the other position index o inside source chunk sc: own chunk forward o = j <= t, dV
+  // o = t >= j; any other source chunk is live as a whole
+  auto ob_range = [&](int sc, int& lo, int& hi) {
+    lo = (IS_DV && sc == c) ? 2 * nh : 0;
+    hi = (!IS_DV && sc == c) ? 2 * (nh + 1) : 4;
+  };
 
   // ---- phase 0: resident rows, gate vectors (and n_prev) into LDS; first score slab into registers
   constexpr int KV = 128 * 8 / NTH;  // 16-byte vectors per thread per score slab (128 rows x 64 columns)
   uint4 kreg[KV];
-  auto load_kslab = [&](int slab) {
+  // Streamed rows are addressed as a uniform base plus a 32-bit byte offset per lane (offsets inside one (batch, head)
+  // fit 32 bits, checked by the launcher), which keeps the addresses out of the vector registers.  Rows past the end
+  // of the sequence are read from its last row instead of being zeroed: their gate factor is zero (forward) or the
+  // value rows they meet are stored as zeros (dV), and rows of dead blocks only feed score units nobody reads.
+  const char* const Xo_b = (const char*)Xo_g;
+  const char* const Xw_b = (const char*)Xw_g;
+  auto load_kslab = [&](int sc, int slab) {
+    const int tv = opaque(tid);
+    const uint32_t krow0 = tv >> 3, kunit = (tv & 7) * 16;
 #pragma unroll
     for (int v = 0; v < KV; ++v) {
-      const int idx = tid + v * NTH;
-      const int j = idx >> 3, cv = idx & 7;
-      const int t = t_base + j;
-      const bool live = j >= 32 * ob_lo && j < 32 * ob_hi && t < S;
-      kreg[v] = live ? *(const uint4*)(Xo_g + (size_t)t * DHQK + slab * 64 + cv * 8) : make_uint4(0, 0, 0, 0);
+      const uint32_t t = min((uint32_t)(sc * kChunk) + krow0 + v * (NTH / 8), (uint32_t)(S - 1));
+      kreg[v] = *(const uint4*)(Xo_b + (t * (uint32_t)(DHQK * 2) + (uint32_t)(slab * 128) + kunit));
     }
   };
-  load_kslab(0);
+  load_kslab(sc_lo, 0);
   // state fragments of the first contraction steps of the first column tile: requested up front, together with
-  // everything else this workgroup needs first, so that all of it costs ONE trip to memory (they are consumed in
-  // the main phase, after the score phase)
+  // everything else this workgroup needs first, so that all of it costs ONE trip to memory
   const int m_wave = wave * MW;  // first value column of this wave inside a column tile
   const int ND = DHQK / 16;
-  const uint4* const st_chunk = (const uint4*)a.states + ((size_t)bh * NC + c) * (size_t)(DHHV / 32) * ND * 64 + lane;
+  const int NCS = (NC + stride - 1) / stride;
+  const char* const st_chunk = (const char*)((const uint4*)a.states + ((size_t)bh * NCS + slot) * (size_t)(DHHV / 32) * ND * 64);
   Frag ring[PD][MB];
-#define MLSTM_LOAD_RING(wt_, stride_)                                                                      \
+  // state fragments of value columns col_ .. col_ + 31 (fragment block col_ / 32), contraction step ds_
+#define MLSTM_STATE_FRAG(col_, ds_) \
+  (*(const uint4*)(st_chunk + (size_t)(((col_) / 32) * ND + (ds_)) * 1024 + st_lane))
+#define MLSTM_LOAD_RING(col0_)                                                                             \
   {                                                                                                        \
-    const uint4* s0_ = st_chunk + ((size_t)((wt_) * WT + m_wave) / 32 * ND) * 64;                          \
+    const uint32_t st_lane = opaque(lane) * 16;                                                            \
     _Pragma("unroll") for (int p = 0; p < PD; ++p)                                                         \
       _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                                                    \
-        ring[p][mb].u = s0_[(size_t)(mb * ND + p) * (stride_)];                                            \
+        ring[p][mb].u = MLSTM_STATE_FRAG((col0_) + m_wave + 32 * mb, p);                                   \
   }
-  MLSTM_LOAD_RING(0, 64)
+  MLSTM_LOAD_RING(0)
   {
     // resident rows: all loads of a batch are issued before the first LDS store (a load-store-load-store loop
     // would pay the memory latency once per iteration)
@@ -139,310 +162,379 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         if (idx < 64 * vec_per_row) store_perm16(Ns + j * QS, cv, make_uint4(qrow[u][0], qrow[u][1], qrow[u][2], qrow[u][3]));
       }
     }
-    for (int idx = tid; idx < 128; idx += NTH) {
-      uu[idx] = a.g.u[gofs + idx];
-      ww[idx] = a.g.w[gofs + idx];
-      if (IS_DV) inv[idx] = a.use_nrow ? 1.f / (a.nrow[gofs + idx] + a.eps) : 1.f;
+    if (tid < 64) {
+      // weight of the kept boundary state for this chunk: the decay over the chunks between the boundary and this
+      // one, re-stabilised (1 when the boundary is the chunk's own)
+      float gsum = 0.f, xs;
+      if (IS_DV) {
+        for (int x = c + 1; x <= sc_hi; ++x) gsum += graw[x];
+        xs = sc_hi > c ? __expf(gsum + mst[c + 1] - mst[sc_hi + 1]) : 1.f;
+      } else {
+        for (int x = sc_lo; x < c; ++x) gsum += graw[x];
+        xs = sc_lo < c ? __expf(gsum + mst[sc_lo] - mst[c]) : 1.f;
+      }
+      const float base = IS_DV ? a.g.abar[gofs + n0 + tid] : a.g.bbar[gofs + n0 + tid] * a.qk_scale;
+      cs[tid] = base * xs;
+      nvec[tid] = IS_DV ? a.g.w[gofs + n0 + tid] : a.g.u[gofs + n0 + tid];
+      if (!IS_DV) {
+        cs0[tid] = base;
+        // fetched with everything else: read from global memory in the denominator phase, the stabiliser costs that
+        // phase a whole trip to memory
+        mcs[tid] = a.g.mcomb[gofs + n0 + tid];
+      }
     }
-    for (int idx = tid; idx < 64; idx += NTH)
-      cs[idx] = IS_DV ? a.g.abar[gofs + n0 + idx] : a.g.bbar[gofs + n0 + idx] * a.qk_scale;
     if (!IS_DV) {
       for (int d = tid; d < DHQK; d += NTH) nperm[perm16(d)] = a.nstates[((size_t)bh * NC + c) * DHQK + d];
-      // fetched with everything else: read from global memory in the denominator phase, the stabiliser costs that
-      // phase a whole trip to memory
-      for (int idx = tid; idx < 64; idx += NTH) mcs[idx] = a.g.mcomb[gofs + n0 + idx];
     }
   }
 
-  MLSTM_PTICK(0)
-  // ---- phase S: score units (32 o x 32 n; unit u = block ob_lo + u/2, position block u%2), dealt round-robin to the
-  // waves; contraction over DHQK in slabs of 64
   constexpr int UW = 8 / NWAVE;  // score units per wave
-  f32x16 sacc[UW];
-#pragma unroll
-  for (int k = 0; k < UW; ++k)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[k][i] = 0.f;
-  const int nslab = DHQK / 64;
-  for (int slab = 0; slab < nslab; ++slab) {
-    __syncthreads();  // previous slab fully consumed (and phase-0 writes visible on the first pass)
-#pragma unroll
-    for (int v = 0; v < KV; ++v) {
-      const int idx = tid + v * NTH;
-      store_perm16(Ts + (idx >> 3) * KS, idx & 7, kreg[v]);
-    }
-    __syncthreads();
-    if (slab + 1 < nslab) load_kslab(slab + 1);
-#pragma unroll
-    for (int k = 0; k < UW; ++k) {
-      // unconditional on purpose: a wave whose block lies above the diagonal multiplies zero rows (its result is
-      // dropped at the gating step); a branch here would make the compiler shuttle the score accumulators between
-      // the two register files on every iteration
-      const int u = wave + k * NWAVE;
-      const int ob = ob_lo + (u >> 1), nb = u & 1;
-      const int obc = ob < 4 ? ob : 3;
-#pragma unroll
-      for (int ds = 0; ds < 4; ++ds) {
-        Frag A, B;
-        A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);
-        B.u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
-        mfma32(sacc[k], A, B);
-      }
-    }
-  }
-  MLSTM_PTICK(1)
-  // first value slab into registers while the score matrix is gated
-  constexpr int VV = 32 * (WT / 8) / NTH;  // 16-byte vectors per thread per value slab (32 rows x WT columns)
+  constexpr int VV = VR * (GW / 8) / NTH;  // 16-byte vectors per thread per value slab (VR rows x GW columns)
+  static_assert(VV >= 1, "value slab smaller than the workgroup");
   uint4 vreg[VV];
-  auto load_vslab = [&](int wt, int ob) {
+  auto load_vslab = [&](int grp, int sc, int sl) {
+    const int tv = opaque(tid);
+    const uint32_t vrow0 = tv / (GW / 8), vunit = (tv % (GW / 8)) * 16;
 #pragma unroll
     for (int v = 0; v < VV; ++v) {
-      const int idx = tid + v * NTH;
-      const int j = idx / (WT / 8), cv = idx % (WT / 8);
-      const int t = t_base + 32 * ob + j;
-      vreg[v] = t < S ? *(const uint4*)(Xw_g + (size_t)t * DHHV + wt * WT + cv * 8) : make_uint4(0, 0, 0, 0);
+      const uint32_t t = min((uint32_t)(sc * kChunk + VR * sl) + vrow0 + v * (NTH / (GW / 8)), (uint32_t)(S - 1));
+      vreg[v] = *(const uint4*)(Xw_b + (t * (uint32_t)(DHHV * 2) + (uint32_t)(grp * GW * 2) + vunit));
     }
   };
-  load_vslab(0, ob_lo);
-  // gate, mask, round, and write P as Ps[n][o]; forward also accumulates fp32 row sums over j
-#pragma unroll
-  for (int k = 0; k < UW; ++k) {
-    const int u = wave + k * NWAVE;
-    const int ob = ob_lo + (u >> 1), nb = u & 1;
-    float rsum = 0.f;
-    if (ob < ob_hi) {
-      const int nl = 32 * nb + r;    // position inside this workgroup's half
-      const int n = n0 + nl;         // position inside the chunk
-      const float un = IS_DV ? ww[n] : uu[n];  // dV: n is the key position j -> w_j ; forward: n = t -> u_t
-#pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int o0 = 32 * ob + 8 * g4 + 4 * h;
-        const float4 xo = *(const float4*)((IS_DV ? uu : ww) + o0);
-        const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
-        float rho[4] = {1.f, 1.f, 1.f, 1.f};
-        if (IS_DV) {
-          const float4 rr = *(const float4*)(inv + o0);
-          rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
-        }
-        float pv[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // exponent u_t - w_j and causal mask j <= t
-          const float ex = IS_DV ? (xov[e] - un) : (un - xov[e]);
-          const bool keep = IS_DV ? (n <= o0 + e) : (o0 + e <= n);
-          const float val = sacc[k][4 * g4 + e] * a.qk_scale * __expf(ex) * rho[e];
-          pv[e] = keep ? val : 0.f;
-          rsum += pv[e];
-        }
-        *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
-      }
-    }
-    if (!IS_DV) {
-      const float tot = rsum + __shfl_xor(rsum, 32);
-      if (h == 0) rows[u * 32 + r] = tot;  // units above the diagonal publish zero
-    }
-  }
-  __syncthreads();
+  const int nslab = DHQK / 64;
 
-  MLSTM_PTICK(2)
-  // ---- phase D (forward): denominators; NTH/64 threads share a row
-  if (!IS_DV) {
-    constexpr int TPR = NTH / 64;  // threads per row: 8, 4, 2 or 1
-    const int t = tid / TPR, part = tid % TPR;
-    const int seg = DHQK / TPR;
-    const uint16_t* qrow = Ns + t * QS + part * seg;
-    const float* np = nperm + part * seg;
-    float dot = 0.f;
-    for (int d = 0; d < seg; d += 8) {
-      const uint4 qv = *(const uint4*)(qrow + d);
-      const uint32_t qq[4] = {qv.x, qv.y, qv.z, qv.w};
+  for (int grp = 0; grp < NG; ++grp) {
+    f32x16 acc[NTG][MB][2];
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        dot += __uint_as_float(qq[p] << 16) * np[d + 2 * p];
-        dot += __uint_as_float(qq[p] & 0xffff0000u) * np[d + 2 * p + 1];
-      }
-    }
+    for (int tl = 0; tl < NTG; ++tl)
 #pragma unroll
-    for (int o = TPR / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
-    if (part == 0) {
-      float nmax = 1.f, iv = 1.f;
-      if (a.use_nrow) {
-        float den = cs[t] * dot;
+      for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-        for (int ob4 = 0; ob4 < 4; ++ob4) den += rows[(2 * ob4 + (t >> 5)) * 32 + (t & 31)];
-        const float mc = mcs[t];
-        const float floor_v = a.sig_gate ? 1.f : __expf(-mc);
-        nmax = fmaxf(fabsf(den), floor_v);
-        iv = 1.f / (nmax + a.eps);
-      }
-      inv[t] = iv;
-      {
-        a.nrow_out[gofs + n0 + t] = nmax;
-        const int tg = t_base + n0 + t;
-        if (tg < S) {
-          if (a.n_out != nullptr) a.n_out[(size_t)bh * S + tg] = nmax;
-          if (a.m_out != nullptr) a.m_out[(size_t)bh * S + tg] = mcs[t];
-        }
-      }
-    }
-  }
-
-  MLSTM_PTICK(3)
-  // ---- main phase, once per column tile: Out^T = (State^T Xn^T) * colscale + Xw^T P.  The resident rows, the gated
-  // score matrix and the denominators above are shared by all column tiles of this (chunk, position half).
-  const int q16 = (lane >> 4) & 1, i16 = lane & 15;
-  const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
-  for (int wt = 0; wt < NWT; ++wt) {
-    f32x16 acc[MB][2];
+        for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+          for (int i = 0; i < 16; ++i) acc[tl][mb][nb][i] = 0.f;
+    __syncthreads();  // phase-0 writes visible (later groups: the previous group's output staging is stored)
+    // ---- inter-chunk product, tile by tile: Out^T = State^T Xn^T
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
-    {
-      const uint4* s0 = st_chunk + ((size_t)(wt * WT + m_wave) / 32 * ND) * 64;
+    for (int tl = 0; tl < NTG; ++tl) {
+      const int col0 = grp * GW + tl * WT;
       for (int ds0 = 0; ds0 < ND; ds0 += PD) {
+        const int ln = opaque(lane);
+        const int r = ln & 31, h = ln >> 5;
+        const uint32_t st_lane = ln * 16;
 #pragma unroll
         for (int p = 0; p < PD; ++p) {
           const int ds = ds0 + p;
           Frag A[MB], B[2];
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb) A[mb] = ring[p][mb];
-          if (ds + PD < ND) {
+          {
+            // unconditional (the last PD steps re-request the tile's last fragment, a cache hit): a conditional load
+            // makes the compiler park ring registers in scratch memory, with a full wait for the load behind it
+            const int dn = min(ds + PD, ND - 1);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) ring[p][mb].u = s0[(size_t)(mb * ND + ds + PD) * 64];
+            for (int mb = 0; mb < MB; ++mb) ring[p][mb].u = MLSTM_STATE_FRAG(col0 + m_wave + 32 * mb, dn);
           }
 #pragma unroll
           for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ns + (32 * nb + r) * QS + 16 * ds + 8 * h);
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
+            for (int nb = 0; nb < 2; ++nb) mfma32(acc[tl][mb][nb], A[mb], B[nb]);
         }
       }
-    }
-    // the next column tile's first state fragments travel while this tile finishes.  The load is unconditional (a
-    // conditional one makes the compiler spill ring registers); after the last tile every ring slot re-requests one
-    // and the same fragment (stride 0), which costs a cache hit instead of 64 KB of fetches from HBM.
-    {
-      const bool more_tiles = wt + 1 < NWT;
-      const int wt_next = more_tiles ? wt + 1 : wt;
-      const int ring_stride = more_tiles ? 64 : 0;
-      MLSTM_LOAD_RING(wt_next, ring_stride)
+      // the next tile's first state fragments travel while this one finishes
+      if (tl + 1 < NTG) MLSTM_LOAD_RING(col0 + WT)
     }
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const float sc = cs[32 * nb + r];
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) acc[mb][nb] *= sc;
-    }
-    MLSTM_PTICK(4)
-    for (int ob = ob_lo; ob < ob_hi; ++ob) {
-      __syncthreads();  // slab buffer free (first pass: P / inv written, score slabs consumed; later: staging stored)
+      for (int tl = 0; tl < NTG; ++tl)
 #pragma unroll
-      for (int v = 0; v < VV; ++v) {
-        const int idx = tid + v * NTH;
-        *(uint4*)(Ts + (idx / (WT / 8)) * VS + (idx % (WT / 8)) * 8) = vreg[v];
+        for (int mb = 0; mb < MB; ++mb) acc[tl][mb][nb] *= sc;
+    }
+
+    // ---- source chunks: score block, gated into Ps, then Out^T += Xw^T P for every value column of the group
+    for (int sc = sc_lo; sc <= sc_hi; ++sc) {
+      int ob_lo, ob_hi;
+      ob_range(sc, ob_lo, ob_hi);
+      const bool own = sc == c;
+      // decay between the key chunk and the query chunk of this block (0 for the own chunk)
+      float gs = 0.f;
+      for (int x = (IS_DV ? c : sc); x < (IS_DV ? sc : c); ++x) gs += graw[x];
+      // gate vectors of the source chunk: requested now, published before the first barrier of the slab loop
+      constexpr int OVN = NTH >= 128 ? 1 : 128 / NTH;  // gate-vector entries per thread (a workgroup may be one wave)
+      float ov[OVN], orh[OVN];
+#pragma unroll
+      for (int e = 0; e < OVN; ++e) {
+        const int idx = tid + e * NTH;
+        ov[e] = 0.f;
+        orh[e] = 1.f;
+        if (idx < 128) {
+          ov[e] = (IS_DV ? a.g.u : a.g.w)[hofs + (size_t)sc * kChunk + idx];
+          if (IS_DV && a.use_nrow) orh[e] = a.nrow[hofs + (size_t)sc * kChunk + idx];
+        }
+      }
+      // score units (32 o x 32 n; unit u = block ob_lo + u/2, position block u%2), dealt round-robin to the waves;
+      // contraction over DHQK in slabs of 64
+      f32x16 sacc[UW];
+#pragma unroll
+      for (int k = 0; k < UW; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sacc[k][i] = 0.f;
+      for (int slab = 0; slab < nslab; ++slab) {
+        const int tv = opaque(tid);
+        const int r = tv & 31, h = (tv >> 5) & 1;
+        __syncthreads();  // previous slab / previous value slab / output staging fully consumed
+#pragma unroll
+        for (int v = 0; v < KV; ++v) {
+          const int idx = tv + v * NTH;
+          store_perm16(Ts + (idx >> 3) * KS, idx & 7, kreg[v]);
+        }
+        if (slab == 0) {
+#pragma unroll
+          for (int e = 0; e < OVN; ++e) {
+            const int idx = tv + e * NTH;
+            if (idx < 128) {
+              ovec[idx] = ov[e];
+              if (IS_DV) orho[idx] = a.use_nrow ? 1.f / (orh[e] + a.eps) : 1.f;
+            }
+          }
+        }
+        __syncthreads();
+        if (slab + 1 < nslab) load_kslab(sc, slab + 1);
+#pragma unroll
+        for (int k = 0; k < UW; ++k) {
+          // unconditional on purpose: a wave whose block lies above the diagonal multiplies zero rows (its result is
+          // dropped at the gating step); a branch here would make the compiler shuttle the score accumulators between
+          // the two register files on every iteration
+          const int u = wave + k * NWAVE;
+          const int ob = ob_lo + (u >> 1), nb = u & 1;
+          const int obc = ob < 4 ? ob : 3;
+#pragma unroll
+          for (int ds = 0; ds < 4; ++ds) {
+            Frag A, B;
+            A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);
+            B.u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
+            mfma32(sacc[k], A, B);
+          }
+        }
+      }
+      // first value slab into registers while the score block is gated
+      load_vslab(grp, sc, ob_lo * (32 / VR));
+      // gate, mask, round, and write P as Ps[n][o]; forward also accumulates fp32 row sums over j of the own chunk
+      const int lg = opaque(lane);
+#pragma unroll
+      for (int k = 0; k < UW; ++k) {
+        const int r = lg & 31, h = lg >> 5;
+        const int u = wave + k * NWAVE;
+        const int ob = ob_lo + (u >> 1), nb = u & 1;
+        float rsum = 0.f;
+        if (ob < ob_hi) {
+          const int nl = 32 * nb + r;    // position inside this workgroup's half
+          const int n = n0 + nl;         // position inside the chunk
+          const float un = nvec[nl] + (IS_DV ? -gs : gs);
+#pragma unroll
+          for (int g4 = 0; g4 < 4; ++g4) {
+            const int o0 = 32 * ob + 8 * g4 + 4 * h;
+            const float4 xo = *(const float4*)(ovec + o0);
+            const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
+            float rho[4] = {1.f, 1.f, 1.f, 1.f};
+            if (IS_DV) {
+              const float4 rr = *(const float4*)(orho + o0);
+              rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
+            }
+            float pv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              // exponent u_t - w_j (+ the decay between the chunks) and, in the own chunk, the causal mask j <= t
+              const float ex = IS_DV ? (xov[e] - un) : (un - xov[e]);
+              const bool keep = !own || (IS_DV ? (n <= o0 + e) : (o0 + e <= n));
+              const float val = sacc[k][4 * g4 + e] * a.qk_scale * __expf(ex) * rho[e];
+              pv[e] = keep ? val : 0.f;
+              rsum += pv[e];
+            }
+            *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+          }
+        }
+        if (!IS_DV && own && grp == 0) {
+          const float tot = rsum + __shfl_xor(rsum, 32);
+          if (h == 0) rows[u * 32 + r] = tot;  // units above the diagonal publish zero
+        }
       }
       __syncthreads();
-      {
-        // next slab of this tile, or the first slab of the next tile (the very last one re-requests itself)
-        const bool more = ob + 1 < ob_hi;
-        const int wt_n = more ? wt : (wt + 1 < NWT ? wt + 1 : wt);
-        load_vslab(wt_n, more ? ob + 1 : ob_lo);
-      }
+
+      // ---- denominators (forward, own chunk = last source chunk, first group only); NTH/64 threads share a row
+      if (!IS_DV && own && grp == 0) {
+        constexpr int TPR = NTH / 64;  // threads per row: 8, 4, 2 or 1
+        const int td = opaque(tid);
+        const int t = td / TPR, part = td % TPR;
+        const int seg = DHQK / TPR;
+        const uint16_t* qrow = Ns + t * QS + part * seg;
+        const float* np = nperm + part * seg;
+        float dot = 0.f;
+        for (int d = 0; d < seg; d += 8) {
+          const uint4 qv = *(const uint4*)(qrow + d);
+          const uint32_t qq[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
-      for (int jl = 0; jl < 2; ++jl) {
-        Frag A[MB], B[2];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const uint16_t* p = Ts + (16 * jl + krow) * VS + (m_wave + 32 * mb + ncol);
-          A[mb].d[0] = lds_read_tr16(p);
-          A[mb].d[1] = lds_read_tr16(p + 4 * VS);
+          for (int p = 0; p < 4; ++p) {
+            dot += __uint_as_float(qq[p] << 16) * np[d + 2 * p];
+            dot += __uint_as_float(qq[p] & 0xffff0000u) * np[d + 2 * p + 1];
+          }
         }
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + 32 * ob + 16 * jl + 8 * h);
+        for (int o = TPR / 2; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
+        if (part == 0) {
+          float nmax = 1.f, iv = 1.f;
+          if (a.use_nrow) {
+            float den = cs0[t] * dot;
+#pragma unroll
+            for (int ob4 = 0; ob4 < 4; ++ob4) den += rows[(2 * ob4 + (t >> 5)) * 32 + (t & 31)];
+            const float mc = mcs[t];
+            const float floor_v = a.sig_gate ? 1.f : __expf(-mc);
+            nmax = fmaxf(fabsf(den), floor_v);
+            iv = 1.f / (nmax + a.eps);
+          }
+          inv[t] = iv;
+          a.nrow_out[gofs + n0 + t] = nmax;
+          const int tg = t_base + n0 + t;
+          if (tg < S) {
+            if (a.n_out != nullptr) a.n_out[(size_t)bh * S + tg] = nmax;
+            if (a.m_out != nullptr) a.m_out[(size_t)bh * S + tg] = mcs[t];
+          }
+        }
+      }
+
+      // ---- Out^T += Xw^T P over the live rows of the source chunk, VR rows per slab
+      const int sl_lo = ob_lo * (32 / VR), sl_hi = ob_hi * (32 / VR);
+      for (int sl = sl_lo; sl < sl_hi; ++sl) {
+        const int tv = opaque(tid);
+        const int ln = tv & 63;
+        const int r = ln & 31, h = ln >> 5;
+        const int q16 = (ln >> 4) & 1, i16 = ln & 15;
+        const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
+        __syncthreads();  // slab buffer free (first pass: P written, score slabs consumed)
+#pragma unroll
+        for (int v = 0; v < VV; ++v) {
+          const int j = tv / (GW / 8) + v * (NTH / (GW / 8));
+          const bool inside = sc * kChunk + VR * sl + j < S;
+          *(uint4*)(Ts + j * VS + (tv % (GW / 8)) * 8) = inside ? vreg[v] : make_uint4(0, 0, 0, 0);
+        }
+        __syncthreads();
+        if (sl + 1 < sl_hi) {
+          load_vslab(grp, sc, sl + 1);
+        } else if (sc < sc_hi) {
+          load_kslab(sc + 1, 0);     // first score slab of the next source chunk
+        } else if (grp + 1 < NG) {
+          load_kslab(sc_lo, 0);      // next group starts over with the first source chunk
+        }
+#pragma unroll
+        for (int jl = 0; jl < JL; ++jl) {
+          Frag B[2];
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + VR * sl + 16 * jl + 8 * h);
+#pragma unroll
+          for (int tl = 0; tl < NTG; ++tl) {
+            Frag A[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+              const uint16_t* p = Ts + (16 * jl + krow) * VS + (tl * WT + m_wave + 32 * mb + ncol);
+              A[mb].d[0] = lds_read_tr16(p);
+              A[mb].d[1] = lds_read_tr16(p + 4 * VS);
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+              for (int nb = 0; nb < 2; ++nb) mfma32(acc[tl][mb][nb], A[mb], B[nb]);
+          }
+        }
+      }
+    }
+
+    // The next group's first state fragments travel during the epilogue (held across the score and value phases they
+    // would cost the registers those need).  Unconditional: after the last group the fragments of that group are
+    // requested once more, cache hits nobody waits for; a conditional load would be parked in scratch memory.
+    MLSTM_LOAD_RING(min(grp + 1, NG - 1) * GW)
+    // ---- epilogue: (normalise,) round, transpose through the slab buffer (32 positions at a time), coalesced store
+#pragma unroll
+    for (int tl = 0; tl < NTG; ++tl) {
+      uint16_t* Og = a.Out + (size_t)bh * S * DHHV + grp * GW + tl * WT;
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const int le = opaque(lane);
+        const int r = le & 31, h = le >> 5;
+        __syncthreads();  // slab buffer free (last value slab consumed / previous half stored; inv written)
+        const float iv = IS_DV ? 1.f : inv[32 * nb + r];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
-      }
-    }
-    MLSTM_PTICK(5)
-
-    // ---- epilogue: (normalise,) round, transpose through the slab buffer (32 positions at a time), coalesced store
-    uint16_t* Og = a.Out + (size_t)bh * S * DHHV + wt * WT;
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      __syncthreads();  // slab buffer free (last value slab consumed / previous half stored)
-      const float iv = IS_DV ? 1.f : inv[32 * nb + r];
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
-          *(uint2*)(Ts + r * HS + w0) =
-              make_uint2(pack_bf16x2(acc[mb][nb][4 * g4 + 0] * iv, acc[mb][nb][4 * g4 + 1] * iv),
-                         pack_bf16x2(acc[mb][nb][4 * g4 + 2] * iv, acc[mb][nb][4 * g4 + 3] * iv));
+          for (int g4 = 0; g4 < 4; ++g4) {
+            const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
+            *(uint2*)(Ts + r * HS + w0) =
+                make_uint2(pack_bf16x2(acc[tl][mb][nb][4 * g4 + 0] * iv, acc[tl][mb][nb][4 * g4 + 1] * iv),
+                           pack_bf16x2(acc[tl][mb][nb][4 * g4 + 2] * iv, acc[tl][mb][nb][4 * g4 + 3] * iv));
+          }
+        __syncthreads();
+        constexpr int vec_per_row = WT / 8;
+        for (int idx = opaque(tid); idx < 32 * vec_per_row; idx += NTH) {
+          const int j = idx / vec_per_row, cv = idx % vec_per_row;
+          const int t = t_base + n0 + 32 * nb + j;
+          // non-temporal: nobody in this launch reads the output, it should not evict shared operands from the L2
+          if (t < S) __builtin_nontemporal_store(*(const u32x4*)(Ts + j * HS + cv * 8), (u32x4*)(Og + (size_t)t * DHHV + cv * 8));
         }
-      __syncthreads();
-      constexpr int vec_per_row = WT / 8;
-      for (int idx = tid; idx < 32 * vec_per_row; idx += NTH) {
-        const int j = idx / vec_per_row, cv = idx % vec_per_row;
-        const int t = t_base + n0 + 32 * nb + j;
-        // non-temporal: nobody in this launch reads the output, it should not evict shared operands from the L2
-        if (t < S) __builtin_nontemporal_store(*(const u32x4*)(Ts + j * HS + cv * 8), (u32x4*)(Og + (size_t)t * DHHV + cv * 8));
       }
     }
   }
 #undef MLSTM_LOAD_RING
-  MLSTM_PTICK(6)
-#ifdef MLSTM_PAR_TIMING
-  if (blk.y == a.NC / 2 && blk.z == 0 && lane == 0)
-    for (int p = 0; p < 7; ++p) a.timing[(blk.x * 4 + (wave & 3)) * 8 + p] = tph[p];
-#endif
+#undef MLSTM_STATE_FRAG
 }
 
-template <int WT, bool IS_DV, int PD, int MW>
+template <int WT, int NTG, bool IS_DV, int PD, int MW>
 __global__ __launch_bounds__(64 * (WT / MW))
     __attribute__((amdgpu_waves_per_eu(PAR_HV_WPE(WT, MW), PAR_HV_WPE(WT, MW)))) void par_hv_kernel(ParHvArgs a) {
-  par_hv_body<WT, IS_DV, PD, MW>(a, xcd_block_id());  // both halves of a chunk share operands: same XCD
+  par_hv_body<WT, NTG, IS_DV, PD, MW>(a, xcd_block_id());  // the workgroups that share a kept state run on one XCD
 }
 
-template <int WT, bool IS_DV, int PD, int MW>
+template <int WT, int NTG, bool IS_DV, int PD, int MW>
 static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
+  constexpr int GW = WT * NTG;
+  constexpr int VR = GW > 256 ? 16 : 32;
   const int QS = a.DHQK + 8;
   const size_t n_region = (size_t)64 * QS;
-  const size_t t_region = (128 * 72 > 32 * (WT + 32)) ? 128 * 72 : 32 * (WT + 32);
-  const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(128 * 3 + 64 + 8 * 32 + a.DHQK + 64) * 4;
+  const size_t t_region = (128 * 72 > VR * (GW + 32)) ? 128 * 72 : VR * (GW + 32);
+  const size_t smem = (n_region + 64 * 136 + t_region) * 2 + (size_t)(64 + 128 * 2 + 64 * 2 + 8 * 32 + a.DHQK + 64 * 2) * 4;
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
-  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, IS_DV, PD, MW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if ((size_t)a.S * (size_t)(a.DHHV > a.DHQK ? a.DHHV : a.DHQK) * 2 >= ((size_t)1 << 32))
+    return "par_hv: one (batch, head) slab of an input exceeds 4 GiB";
+  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, NTG, IS_DV, PD, MW>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_hv: cannot raise the dynamic LDS limit";
   dim3 grid(2, a.NC, BH);
-  hipLaunchKernelGGL((par_hv_kernel<WT, IS_DV, PD, MW>), grid, dim3(64 * (WT / MW)), smem, stream, a);
+  hipLaunchKernelGGL((par_hv_kernel<WT, NTG, IS_DV, PD, MW>), grid, dim3(64 * (WT / MW)), smem, stream, a);
   return nullptr;
 }
 
-template <int WT, bool IS_DV>
+template <int WT, int NTG, bool IS_DV>
 static const char* launch_par_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
   // eight steps ahead (64 registers of fragments in flight per lane) measured 8 % faster than four at 256/512
-  constexpr int MW = WT == 256 ? MLSTM_PAR_HV_MW256 : 64;
-  if (a.DHQK % 128 == 0) return launch_par_hv_pd<WT, IS_DV, 8, MW>(a, BH, stream);
-  return launch_par_hv_pd<WT, IS_DV, 4, MW>(a, BH, stream);
+  constexpr int MW = WT == 256 ? 32 : 64;
+  if (a.DHQK % 128 == 0) return launch_par_hv_pd<WT, NTG, IS_DV, 8, MW>(a, BH, stream);
+  return launch_par_hv_pd<WT, NTG, IS_DV, 4, MW>(a, BH, stream);
+}
+
+template <bool IS_DV>
+static const char* launch_par_hv_d(const ParHvArgs& a, int BH, hipStream_t stream) {
+  if (a.DHHV % 512 == 0) return launch_par_hv_t<256, 2, IS_DV>(a, BH, stream);
+  if (a.DHHV % 256 == 0) return launch_par_hv_t<256, 1, IS_DV>(a, BH, stream);
+  if (a.DHHV % 128 == 0) return launch_par_hv_t<128, 1, IS_DV>(a, BH, stream);
+  return launch_par_hv_t<64, 1, IS_DV>(a, BH, stream);
 }
 
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
   if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "par_hv: DHQK and DHHV must be multiples of 64";
-  if (is_dv) {
-    if (a.DHHV % 256 == 0) return launch_par_hv_t<256, true>(a, BH, stream);
-    if (a.DHHV % 128 == 0) return launch_par_hv_t<128, true>(a, BH, stream);
-    return launch_par_hv_t<64, true>(a, BH, stream);
-  }
-  if (a.DHHV % 256 == 0) return launch_par_hv_t<256, false>(a, BH, stream);
-  if (a.DHHV % 128 == 0) return launch_par_hv_t<128, false>(a, BH, stream);
-  return launch_par_hv_t<64, false>(a, BH, stream);
+  if (a.stride < 1 || a.stride > kMaxStateStride) return "par_hv: state stride out of range";
+  return is_dv ? launch_par_hv_d<true>(a, BH, stream) : launch_par_hv_d<false>(a, BH, stream);
 }
 
 }  // namespace mlstm

@@ -142,12 +142,6 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   };
 
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
-#ifdef MLSTM_SCAN_TIMING
-  unsigned long long tph[5] = {0, 0, 0, 0, 0}, tlast = __builtin_amdgcn_s_memtime();
-#define MLSTM_STICK(p_) { const unsigned long long now_ = __builtin_amdgcn_s_memtime(); tph[p_] += now_ - tlast; tlast = now_; }
-#else
-#define MLSTM_STICK(p_)
-#endif
   // row scales of the first chunk straight into the table, those of the second chunk into the prefetch register
   {
     const int t = c_first * kChunk + srow;
@@ -222,16 +216,18 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       *(uint4*)(Yh + j * YS + cv * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
       if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     }
-    MLSTM_STICK(0)
     __syncthreads();
-    MLSTM_STICK(1)
     if (hit + 1 < NC * NP) prefetch(piece + 1 < NP ? c : c + c_step, piece + 1 < NP ? piece + 1 : 0);
     if (piece == 0) load_scales(c + 2 * c_step);
 
-    // ---- emit the state before this chunk's update as bf16 operand fragments
-    if (piece == 0) {
+    // ---- emit the state before this chunk's update as bf16 operand fragments, at the kept boundaries only: forward
+    // the state before every stride-th chunk, backward the gradient of the state after the last chunk of every group
+    // of `stride` chunks (and after the last chunk of the sequence); slot c / stride either way
+    const bool keep = a.backward ? (c == NC - 1 || (c + 1) % a.stride == 0) : (c % a.stride == 0);
+    if (piece == 0 && keep) {
       const size_t ND = DHQK / 16, NW = DHHV / 32;
-      uint4* st = (uint4*)a.states + ((size_t)bh * NC + c) * NW * ND * 64;
+      const size_t NCS = (size_t)(NC + a.stride - 1) / a.stride;
+      uint4* st = (uint4*)a.states + ((size_t)bh * NCS + c / a.stride) * NW * ND * 64;
 #pragma unroll
       for (int db = 0; db < 2; ++db)
 #pragma unroll
@@ -251,7 +247,6 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
           }
         }
     }
-    MLSTM_STICK(2)
     // ---- decay (once per chunk), then accumulate X^T (scale . Y) over the positions of this piece
     const float g = piece == 0 ? gl[it & (kGBlock - 1)] : 1.f;
     if (piece == 0) {
@@ -298,15 +293,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       for (int g2 = 0; g2 < XROWS; ++g2) s += npart[g2 * RT + tid];
       nval = g * nval + s;
     }
-    MLSTM_STICK(3)
     __syncthreads();
-    MLSTM_STICK(4)
   }
-#ifdef MLSTM_SCAN_TIMING
-  if (bx == 0 && by == 0 && bz == 0 && lane == 0)
-    for (int p = 0; p < 5; ++p) a.timing[wave * 8 + p] = tph[p];
-#endif
-
   if (a.final_out != nullptr) {
 #pragma unroll
     for (int db = 0; db < 2; ++db)
@@ -324,10 +312,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
 
 template <int RT, int WT, bool HILO>
 static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
-#ifndef MLSTM_SCAN_FW_WCOLS
-#define MLSTM_SCAN_FW_WCOLS 32
-#endif
-  constexpr int WCOLS = MLSTM_SCAN_FW_WCOLS;
+  constexpr int WCOLS = 32;
   constexpr int NT = 64 * (RT / 64) * (WT / WCOLS);
   constexpr int XROWS = NT / (RT / 8);
   constexpr int PS = 128;
@@ -343,6 +328,7 @@ static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) 
 
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream) {
   if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "scan: DHQK and DHHV must be multiples of 64";
+  if (a.stride < 1 || a.stride > kMaxStateStride) return "scan: state stride out of range";
   const bool r128 = a.DHQK % 128 == 0, w128 = a.DHHV % 128 == 0;
   if (hilo) {
     if (r128 && w128) return launch_scan_t<128, 128, true>(a, BH, stream);

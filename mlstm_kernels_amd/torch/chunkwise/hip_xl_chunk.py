@@ -4,10 +4,18 @@ Mirrors the public operators of the reference,
   mlstm_kernels/torch/chunkwise/triton_xl_chunk/fwbw.py:244-300          (``mlstm_chunkwise__xl_chunk``)
   mlstm_kernels/torch/chunkwise/triton_xl_chunk_siging/fwbw.py:211-269   (``mlstm_siging_chunkwise__xl_chunk``)
 with the same argument names, defaults, return structure and shape rules
-(mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:42-128).  The Triton tile-size keywords are accepted
-and ignored: the HIP kernels always work on internal chunks of 128 positions, which leaves H and the last
-states unchanged because the chunkwise formulation is exact for every chunk length."""
+(mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:42-128).  The HIP kernels always scan the sequence in
+internal chunks of 128 positions (the reference's ``chunk_size_inter``), which leaves H and the last states unchanged
+because the chunkwise formulation is exact for every chunk length.  ``chunk_size_intra`` (a multiple of 128, at most
+1024) selects how far apart the kept chunk states are, as in the reference (``save_states_every_nth_chunk`` =
+``chunk_size_intra // chunk_size_inter``); the Triton tile-size and launch keywords are accepted and ignored.
+
+Arithmetic: the matrix cores multiply bf16 operands and accumulate in fp32; gates, stabilisers, normalisers and
+states are fp32.  float32 and float16 inputs (or ``autocast_kernel_dtype``) are therefore rounded to bfloat16 at the
+boundary -- unlike the reference's Triton kernels, which run in the requested dtype -- and a warning says so once."""
 from __future__ import annotations
+
+import warnings
 
 import torch
 from torch.amp import custom_bwd, custom_fwd
@@ -16,10 +24,41 @@ from ... import _lib
 from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu
 
 _IGNORED_TUNING_KWARGS = (
-    "chunk_size_inter", "chunk_size_intra", "siz_b_L_parallel", "siz_b_L_loop", "siz_b_DH_parallel",
-    "siz_b_DH_loop", "num_warps_intra", "num_warps_inter", "num_stages_intra", "num_stages_inter",
-    "recompute_states_in_bw",
+    "siz_b_L_parallel", "siz_b_L_loop", "siz_b_DH_parallel", "siz_b_DH_loop", "num_warps_intra", "num_warps_inter",
+    "num_stages_intra", "num_stages_inter", "recompute_states_in_bw",
 )
+_INTERNAL_CHUNK = 128
+_warned_rounding: set = set()
+
+
+def _warn_rounding_once(dtype: torch.dtype) -> None:
+    if dtype not in _warned_rounding:
+        _warned_rounding.add(dtype)
+        warnings.warn(
+            f"mlstm_kernels_amd: {dtype} operands are rounded to bfloat16 for the HIP chunkwise kernels (bf16 matrix "
+            "cores with fp32 accumulation; gates, normalisers and states stay fp32). "
+            + ("float16 loses three mantissa bits this way. " if dtype == torch.float16 else "")
+            + "Pass bfloat16 tensors and autocast_kernel_dtype=torch.bfloat16 to make this explicit.",
+            stacklevel=4,
+        )
+
+
+def _state_stride(tuning_kwargs: dict, who: str) -> int:
+    """chunk_size_inter / chunk_size_intra of the reference (kernel_param_heuristics.py:118-121) -> state stride."""
+    for key in tuning_kwargs:
+        if key not in _IGNORED_TUNING_KWARGS and key not in ("chunk_size_inter", "chunk_size_intra"):
+            raise TypeError(f"{who}() got an unexpected keyword argument '{key}'")
+    inter = tuning_kwargs.get("chunk_size_inter")
+    intra = tuning_kwargs.get("chunk_size_intra")
+    if inter is not None and inter != _INTERNAL_CHUNK:
+        raise ValueError(f"the HIP kernels scan in chunks of {_INTERNAL_CHUNK} positions: chunk_size_inter must be "
+                         f"{_INTERNAL_CHUNK} or None, got {inter}")
+    if intra is None:
+        return 0
+    if intra % _INTERNAL_CHUNK != 0 or not (1 <= intra // _INTERNAL_CHUNK <= 8):
+        raise ValueError(f"chunk_size_intra must be a multiple of {_INTERNAL_CHUNK} between {_INTERNAL_CHUNK} and "
+                         f"{8 * _INTERNAL_CHUNK}, got {intra}")
+    return intra // _INTERNAL_CHUNK
 
 
 def _is_pow2(x: int) -> bool:
@@ -37,16 +76,20 @@ def validate_xl_chunk_shapes(S: int, chunk_size: int) -> None:
     assert S % chunk_size == 0, f"Sequence length must be divisible by the target chunk size {chunk_size}."
 
 
-def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep):
+def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep, path, stride):
     B, NH, S, DHQK = q.shape
     DHHV = v.shape[-1]
     dev = q.device
     lib = _lib.get_lib()
-    ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, int(keep))
+    ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, int(keep), path, stride)
     if ws_bytes == 0:
+        if DHQK % 64 == 0 and DHQK > 896:
+            raise RuntimeError(f"DHQK too large for the HIP chunkwise kernels: {DHQK} (at most 896)")
+        if path == _lib.PATH_FUSED and DHQK not in (128, 256) and DHQK % 64 == 0 and DHHV % 64 == 0:
+            raise RuntimeError(f"the fused kernel path supports DHQK = 128 or 256 only, got {DHQK}")
         raise ValueError(
             f"unsupported shape for the HIP chunkwise kernels: B={B}, NH={NH}, S={S}, DHQK={DHQK}, DHHV={DHHV} "
-            "(head dimensions must be multiples of 64, B*NH <= 65535)"
+            "(head dimensions must be multiples of 64, DHQK <= 896, B*NH <= 65535)"
         )
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
@@ -60,7 +103,7 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
         ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0),
         ptr(H), None, None, ptr(c_last), ptr(n_last), ptr(m_last),
         ptr(ws), ws_bytes, int(keep), B, NH, S, DHQK, DHHV, float(eps),
-        _lib.BF16, dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize),
+        _lib.BF16, dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
         current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_chunkwise_fw")
@@ -74,6 +117,9 @@ def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
     assert v.shape[:3] == (B, NH, S), f"v has wrong shape {tuple(v.shape)}"
     assert i.shape == (B, NH, S) and f.shape == (B, NH, S), "i and f must have shape (B, NH, S)"
     bf = torch.bfloat16
+    for t in (q, k, v):
+        if t.dtype != bf:
+            _warn_rounding_once(t.dtype)
     qb, kb, vb = (t.to(bf).contiguous() for t in (q, k, v))
     gate_dt = torch.bfloat16 if (i.dtype == bf and f.dtype == bf) else torch.float32
     ib, fb = i.to(gate_dt).contiguous(), f.to(gate_dt).contiguous()
@@ -89,16 +135,19 @@ def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
     return dev, qb, kb, vb, ib, fb, c0, n0, m0
 
 
-def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool):
+def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, stride: int):
     class _HipChunkwiseFwBw(torch.autograd.Function):
         @staticmethod
         @custom_fwd(device_type="cuda", cast_inputs=autocast_kernel_dtype)
         def forward(ctx, q, k, v, i, f, c0, n0, m0, return_last_states, eps):
+            # outputs nobody differentiates (the last states in most losses) arrive as None in backward instead of as
+            # freshly allocated zero tensors the size of the state
+            ctx.set_materialize_grads(False)
             out_dtype = q.dtype
             dev, qb, kb, vb, ib, fb, c0f, n0f, m0f = _prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
             needs_bw = any(ctx.needs_input_grad[:6])
             H, c_last, n_last, m_last, ws = _fw_launch(
-                qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw
+                qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw, path, stride
             )
             ctx.save_for_backward(qb, kb, vb, ib, fb, ws)
             ctx.cfg = (eps, q.dtype, k.dtype, v.dtype, i.dtype, f.dtype,
@@ -115,8 +164,10 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool):
             DHHV = vb.shape[-1]
             dev = qb.device
             lib = _lib.get_lib()
-            bw_bytes = lib.mlstm_hip_chunkwise_bw_workspace_bytes(B, NH, S, DHQK, DHHV)
+            bw_bytes = lib.mlstm_hip_chunkwise_bw_workspace_bytes(B, NH, S, DHQK, DHHV, stride)
             bws = torch.empty(bw_bytes, dtype=torch.uint8, device=dev)
+            if dH is None:  # only the last states are differentiated
+                dH = torch.zeros(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
             dHb = dH.to(torch.bfloat16).contiguous()
             dCl = None if dC_last is None else dC_last.to(torch.float32).contiguous()
             dQ, dK, dV = torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb)
@@ -127,7 +178,7 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool):
                 ptr(qb), ptr(kb), ptr(vb), ptr(ib), ptr(fb), ptr(dHb), ptr(dCl),
                 ptr(dQ), ptr(dK), ptr(dV), ptr(dI), ptr(dF), ptr(dC0),
                 ptr(ws), ws.numel(), ptr(bws), bw_bytes, B, NH, S, DHQK, DHHV, float(eps),
-                _lib.BF16, dtype_code(ib), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize),
+                _lib.BF16, dtype_code(ib), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
                 current_stream_ptr(dev),
             )
             _lib.check(rc, "mlstm_hip_chunkwise_bw")
@@ -142,12 +193,13 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool):
 _FWBW_CACHE: dict = {}
 
 
-def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool):
+def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool, kernel_path: str, stride: int):
     if autocast_kernel_dtype not in (torch.float32, torch.float16, torch.bfloat16):
         raise ValueError(f"Unsupported kernel dtype {autocast_kernel_dtype}.")
-    key = (autocast_kernel_dtype, siging, normalize)
+    path = _lib.path_code(kernel_path)
+    key = (autocast_kernel_dtype, siging, normalize, path, stride)
     if key not in _FWBW_CACHE:
-        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize)
+        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize, path, stride)
     return _FWBW_CACHE[key]
 
 
@@ -165,19 +217,21 @@ def mlstm_chunkwise__hip_xl_chunk(
     chunk_size: int = 128,
     autocast_kernel_dtype: torch.dtype = torch.float32,
     any_sequence_length: bool = False,
+    kernel_path: str = "auto",
     **tuning_kwargs,
 ):
     """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
     ``(H, (C_last fp32 (B,NH,DHQK,DHHV), n_last fp32 (B,NH,DHQK), m_last fp32 (B,NH,1)))``.
-    The matrix kernels multiply in bf16 with fp32 accumulation whatever the input dtype.
+    The matrix kernels multiply in bf16 with fp32 accumulation whatever the input dtype (other dtypes are rounded to
+    bf16, with a one-time warning).
     ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
-    tail themselves, so every S >= 1 is one call."""
-    for key in tuning_kwargs:
-        if key not in _IGNORED_TUNING_KWARGS:
-            raise TypeError(f"mlstm_chunkwise__hip_xl_chunk() got an unexpected keyword argument '{key}'")
+    tail themselves, so every S >= 1 is one call.  ``kernel_path`` ("auto", "split", "fused"; not in the reference)
+    selects the kernels of the value-column side.  ``chunk_size_intra`` (reference keyword) sets the distance between
+    kept chunk states."""
+    stride = _state_stride(tuning_kwargs, "mlstm_chunkwise__hip_xl_chunk")
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
-    fn = _get_fwbw(autocast_kernel_dtype, False, True)
+    fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride)
     H, c_last, n_last, m_last = fn.apply(q, k, v, i, f, c_initial, n_initial, m_initial, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last, m_last)
@@ -199,16 +253,15 @@ def mlstm_siging_chunkwise__hip_xl_chunk(
     chunk_size: int = 128,
     autocast_kernel_dtype: torch.dtype = torch.float32,
     any_sequence_length: bool = False,
+    kernel_path: str = "auto",
     **tuning_kwargs,
 ):
     """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``.
-    ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules, as for the exp gate."""
-    for key in tuning_kwargs:
-        if key not in _IGNORED_TUNING_KWARGS:
-            raise TypeError(f"mlstm_siging_chunkwise__hip_xl_chunk() got an unexpected keyword argument '{key}'")
+    ``any_sequence_length``, ``kernel_path`` and ``chunk_size_intra`` as for the exp gate."""
+    stride = _state_stride(tuning_kwargs, "mlstm_siging_chunkwise__hip_xl_chunk")
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
-    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize))
+    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride)
     H, c_last, n_last, _ = fn.apply(q, k, v, i, f, c_initial, n_initial, None, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last)

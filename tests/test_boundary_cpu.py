@@ -98,9 +98,17 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in the header but not exported by the library"
     assert lib.mlstm_hip_abi_version() == _lib.ABI_VERSION
     # size queries and argument validation work without a GPU (no kernel is launched)
-    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 64, 128, 1) > 0
-    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 60, 128, 1) == 0
-    assert lib.mlstm_hip_chunkwise_bw_workspace_bytes(1, 2, 256, 64, 128) > 0
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 64, 128, 1, _lib.PATH_AUTO, 0) > 0
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 60, 128, 1, _lib.PATH_AUTO, 0) == 0
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 960, 128, 1, _lib.PATH_AUTO, 0) == 0   # DHQK limit: 896
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 896, 128, 1, _lib.PATH_AUTO, 0) > 0
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 64, 128, 1, _lib.PATH_FUSED, 0) == 0  # fused: 128/256 only
+    assert lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 256, 64, 128, 1, _lib.PATH_AUTO, 9) == 0   # stride 1 .. 8
+    # a chunk state kept every second chunk halves the state part of the workspace
+    full = lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 4096, 256, 512, 1, _lib.PATH_SPLIT, 1)
+    half = lib.mlstm_hip_chunkwise_fw_workspace_bytes(1, 2, 4096, 256, 512, 1, _lib.PATH_SPLIT, 2)
+    assert full - half == 2 * 16 * 256 * 512 * 2
+    assert lib.mlstm_hip_chunkwise_bw_workspace_bytes(1, 2, 256, 64, 128, 0) > 0
     rc = lib.mlstm_hip_step(None, None, None, None, None, None, None, None, None, None, None, None,
                             1, 1, 64, 64, 1e-6, 1, 0, None)
     assert rc != 0 and b"null pointer" in lib.mlstm_hip_last_error()

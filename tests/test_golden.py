@@ -122,14 +122,14 @@ def test_hip_stored_rows_match_reference_native_vectors(case):
     if init:
         c0, n0, m0 = z["c0"].to(dev).contiguous(), z["n0"].to(dev).contiguous(), z["m0"].reshape(B, NH).to(dev).contiguous()
     lib = _lib.get_lib()
-    ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0)
+    ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0, _lib.PATH_AUTO, 0)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
     n_out = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
     m_out = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
     rc = lib.mlstm_hip_chunkwise_fw(ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0), ptr(H), ptr(n_out),
                                     ptr(m_out), None, None, None, ptr(ws), ws_bytes, 0, B, NH, S, DHQK, DHHV, 1e-6,
-                                    _lib.BF16, _lib.F32, _lib.GATE_EXP, 1, current_stream_ptr(dev))
+                                    _lib.BF16, _lib.F32, _lib.GATE_EXP, 1, _lib.PATH_AUTO, 0, current_stream_ptr(dev))
     _lib.check(rc, "mlstm_hip_chunkwise_fw")
     torch.cuda.synchronize()
     assert (m_out.cpu() - z["m_out"]).abs().max() <= 1e-4

@@ -20,29 +20,63 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
-@pytest.fixture(autouse=True, params=["split", "fused"])
-def chunkwise_path(request):
-    """Every test runs once per kernel path of the chunkwise passes: 'split' (state scan + chunk-parallel kernels)
-    and 'fused' (sequential kernels with register-resident state; head dimensions they do not support fall back)."""
-    from mlstm_kernels_amd import _lib
+_VARIANT = {"kernel_path": "auto", "chunk_size_intra": None}
 
-    previous = _lib.set_chunkwise_path(_lib.PATH_SPLIT if request.param == "split" else _lib.PATH_FUSED)
+
+@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "fused-2"])
+def kernel_variant(request):
+    """Every test runs once per kernel variant of the chunkwise passes: the split path (state scan + chunk-parallel
+    kernels) with a chunk state kept every 1, 2 or 4 chunks, and the fused path (sequential kernels with a
+    register-resident state; head dimensions it does not support are skipped)."""
+    path, stride = request.param.split("-")
+    _VARIANT.update(kernel_path=path, chunk_size_intra=128 * int(stride))
     yield request.param
-    _lib.set_chunkwise_path(previous)
+    _VARIANT.update(kernel_path="auto", chunk_size_intra=None)
+
+
+def _with_variant(op):
+    """The chunkwise operator with the kernel variant of the running test filled in."""
+    import functools
+
+    @functools.wraps(op)
+    def call(*args, **kw):
+        kw.setdefault("kernel_path", _VARIANT["kernel_path"])
+        kw.setdefault("chunk_size_intra", _VARIANT["chunk_size_intra"])
+        try:
+            return op(*args, **kw)
+        except RuntimeError as e:
+            if "fused kernel path supports" in str(e):
+                pytest.skip("the fused path does not support these head dimensions")
+            raise
+
+    call.supports_any_sequence_length = True
+    return call
 
 
 def _ops():
     from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk
     from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_sequence__hip, mlstm_recurrent_step__hip
 
-    return mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk, mlstm_recurrent_step__hip, mlstm_recurrent_sequence__hip
+    return (_with_variant(mlstm_chunkwise__hip_xl_chunk), _with_variant(mlstm_siging_chunkwise__hip_xl_chunk),
+            mlstm_recurrent_step__hip, mlstm_recurrent_sequence__hip)
 
 
-def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3):
-    bad = allclose_frac(x, ref, 2e-2, 2e-2)
+def report_offenders(x, ref, name, rtol=2e-2, atol=2e-2):
+    """Prints, for one tensor, how many elements lie outside |x - ref| <= atol + rtol |ref| and the worst error in
+    units of that bound; returns (fraction outside, worst ratio)."""
+    x64, r64 = x.detach().double().cpu(), ref.detach().double().cpu()
+    ratio = (x64 - r64).abs() / (atol + rtol * r64.abs())
+    n_bad, worst = int((ratio > 1).sum()), float(ratio.max())
+    print(f"    {name}: {n_bad} of {ratio.numel()} elements outside {rtol:g}/{atol:g}, worst error {worst:.2f} x the bound")
+    return n_bad / ratio.numel(), worst
+
+
+def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3, worst_tol=12.0):
+    bad, worst = report_offenders(x, ref, name)
     e1, e2 = rel_to_scale(x, ref), rel_norm(x, ref)
-    assert bad <= frac and e1 <= scale_tol and e2 <= norm_tol, (
-        f"{name}: {bad:.2e} of elements outside 2e-2/2e-2, max err / scale {e1:.2e}, norm err {e2:.2e}")
+    assert bad <= frac and worst <= worst_tol and e1 <= scale_tol and e2 <= norm_tol, (
+        f"{name}: {bad:.2e} of elements outside 2e-2/2e-2 (worst {worst:.2f} x the bound), max err / scale {e1:.2e}, "
+        f"norm err {e2:.2e}")
 
 
 def d64(t):
@@ -54,6 +88,8 @@ def d64(t):
     (2, 2, 64, 128), (3, 4, 256, 512), (1, 1, 128, 192),
     (3, 2, 96, 100), (1, 1, 48, 36), (5, 2, 130, 260),   # odd head dimensions: partial slices, ragged row batches
     (40, 8, 256, 512),                                    # 168 MB of state: the cacheable variant at a larger batch
+    (81, 8, 256, 512),                                    # 340 MB of state: the streaming variant, 256-column slices
+    (108, 8, 256, 384),                                   # 340 MB of state: the streaming variant, 128-column slices
 ])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_step_parity(B, NH, DQK, DHV, dtype):
@@ -78,33 +114,39 @@ def test_step_parity(B, NH, DQK, DHV, dtype):
     assert c3.data_ptr() == c_dev.data_ptr() and torch.equal(c3, c2) and torch.equal(h3, h)
 
 
-def test_decode_after_prefill():
-    """Prefill S=2048 with the chunkwise kernel, then 128 consecutive decode steps (state updated in place);
-    the oracle does the same in fp64 for the first two batch rows."""
+@pytest.mark.parametrize("B", [16, 64, 256])
+def test_decode_after_prefill(B):
+    """BASELINE config 5: prefill S=2048 with the chunkwise kernel, then 128 consecutive decode steps (state updated
+    in place) at B = 16, 64 and 256 (the last one streams its 1 GiB state past the caches with the non-temporal
+    kernel variant); the oracle does the same in fp64 for the first and the last batch row.  Inputs are drawn on the
+    GPU (the full-batch tensors are too large to draw on the host) and the checked rows are copied out."""
     exp_op, _, step, _ = _ops()
     from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw
-    B, NH, S, DQK, DHV, T = 16, 8, 2048, 256, 512, 128
-    Bo = 2
-    q, k, v, i, f = make_qkvif(B, NH, S, DQK, DHV, seed=0)
-    _, (c, n, m) = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
-    ref = O.chunkwise_fw(*(d64(t[:Bo]) for t in (q, k, v, i, f)), chunk_size=128)
+    NH, S, DQK, DHV, T = 8, 2048, 256, 512, 128
+    rows = [0, B - 1]
+    gen = torch.Generator(device=DEV).manual_seed(B)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    q, k, v = rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DHV).bfloat16()
+    i, f = rn(B, NH, S), 3 + rn(B, NH, S)
+    with torch.no_grad():
+        _, (c, n, m) = exp_op(q, k, v, i, f, return_last_states=True, chunk_size=128)
+    ref = O.chunkwise_fw(*(d64(t[rows]) for t in (q, k, v, i, f)), chunk_size=128)
+    del q, k, v, i, f
     c_r, n_r, m_r = ref["C_last"], ref["n_last"], ref["m_last"]
-    assert_state_close(c[:Bo], c_r, 1e-3, "prefill C")
-    g = torch.Generator().manual_seed(1)
+    assert_state_close(c[rows], c_r, 1e-3, "prefill C")
     n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
     worst_h = 0.0
     for t in range(T):
-        qt, kt, vt = (torch.randn(B, NH, d, generator=g).bfloat16() for d in (DQK, DQK, DHV))
-        it, ft = torch.randn(B, NH, 1, generator=g), 3 + torch.randn(B, NH, 1, generator=g)
-        h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(c, n, m, qt.to(DEV), kt.to(DEV), vt.to(DEV), it.to(DEV), ft.to(DEV),
-                                                           matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
+        qt, kt, vt = rn(B, NH, DQK).bfloat16(), rn(B, NH, DQK).bfloat16(), rn(B, NH, DHV).bfloat16()
+        it, ft = rn(B, NH, 1), 3 + rn(B, NH, 1)
+        h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(c, n, m, qt, kt, vt, it, ft, matC_new=c, vecN_new=n_alt, scaM_new=m_alt)
         n_alt, m_alt, n, m = n, m, n_new, m_new
-        h_r, (c_r, n_r, m_r) = O.recurrent_step(*(d64(x[:Bo]) for x in (qt, kt, vt, it, ft)), c_r, n_r, m_r)
-        worst_h = max(worst_h, allclose_frac(h[:Bo], h_r, 2e-2, 2e-2))
+        h_r, (c_r, n_r, m_r) = O.recurrent_step(*(d64(x[rows]) for x in (qt, kt, vt, it, ft)), c_r, n_r, m_r)
+        worst_h = max(worst_h, allclose_frac(h[rows], h_r, 2e-2, 2e-2))
     assert worst_h == 0.0, f"h outside 2e-2/2e-2 on a fraction {worst_h} of elements"
-    assert_state_close(c[:Bo], c_r, 1e-3, "C after 128 steps")
-    assert_state_close(n[:Bo], n_r, 1e-3, "n after 128 steps")
-    assert (d64(m[:Bo]) - m_r).abs().max() <= 1e-3
+    assert_state_close(c[rows], c_r, 1e-3, "C after 128 steps")
+    assert_state_close(n[rows], n_r, 1e-3, "n after 128 steps")
+    assert (d64(m[rows]) - m_r).abs().max() <= 1e-3
 
 
 def test_decode_steps_in_hip_graph():
@@ -195,9 +237,10 @@ def test_chunkwise_forward_gate_regimes(f_offset, DQK):
 
 def test_unsupported_head_dim_fails_loudly():
     exp_op, *_ = _ops()
-    q, k, v, i, f = make_qkvif(1, 1, 128, 1024, 128)
-    with pytest.raises(RuntimeError, match="DHQK too large"):
-        exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128)
+    for dqk in (960, 1024):
+        q, k, v, i, f = make_qkvif(1, 1, 128, dqk, 128)
+        with pytest.raises(RuntimeError, match="DHQK too large"):
+            exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128, kernel_path="split")
     q, k, v, i, f = make_qkvif(1, 1, 128, 96, 128)
     with pytest.raises(ValueError, match="multiples of 64"):
         exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128)

@@ -1,5 +1,5 @@
 """Randomised parity sweep: shapes (ragged sequence lengths, head dimensions that are multiples of 64 only), both
-gates, initial states, an upstream dC_last and both chunkwise paths, each against the fp64 oracle.  Tolerances are
+gates, initial states, an upstream dC_last, both chunkwise paths and every state stride, each against the fp64 oracle.  Tolerances are
 norm-relative (bf16 operands): H 6e-3, gradients 8e-3, final C 1e-3 of its scale, gate gradients 5e-2 of theirs."""
 import random
 
@@ -21,12 +21,14 @@ def _case(seed):
         sig=rnd.random() < 0.3, init=rnd.random() < 0.5, dcl=rnd.random() < 0.4,
         f_offset=rnd.choice([0.0, 3.0, 5.0]), fused=rnd.random() < 0.5)
     cfg["normalize"] = (not cfg["sig"]) or rnd.random() < 0.7
+    cfg["stride"] = rnd.choice([1, 2, 3, 4, 8])
+    if cfg["DQ"] not in (128, 256):
+        cfg["fused"] = False   # the fused path supports these two head dimensions only
     return cfg
 
 
-@pytest.mark.parametrize("seed", list(range(16)))
+@pytest.mark.parametrize("seed", list(range(32)))
 def test_random_shape_forward_backward(seed):
-    from mlstm_kernels_amd import _lib
     from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk
 
     c = _case(seed)
@@ -50,19 +52,17 @@ def test_random_shape_forward_backward(seed):
     leaves = [cu(t).requires_grad_(True) for t in (q, k, v, i, f)]
     c0l = None if c0 is None else cu(c0).requires_grad_(True)
     kw = dict(c_initial=c0l, n_initial=cu(n0), m_initial=cu(m0), return_last_states=True, chunk_size=128,
-              any_sequence_length=True)
-    _lib.set_chunkwise_path(_lib.PATH_FUSED if c["fused"] else _lib.PATH_SPLIT)
-    try:
-        if sig:
-            H, st = mlstm_siging_chunkwise__hip_xl_chunk(*leaves, normalize=normalize, **kw)
-        else:
-            H, st = mlstm_chunkwise__hip_xl_chunk(*leaves, **kw)
-        loss = (H.float() * cu(dH).float()).sum()
-        if c["dcl"]:
-            loss = loss + (st[0] * cu(dCl)).sum()
-        loss.backward()
-    finally:
-        _lib.set_chunkwise_path(_lib.PATH_AUTO)
+              any_sequence_length=True, kernel_path="fused" if c["fused"] else "split",
+              chunk_size_intra=128 * c["stride"])
+    print(f"case {c}", flush=True)
+    if sig:
+        H, st = mlstm_siging_chunkwise__hip_xl_chunk(*leaves, normalize=normalize, **kw)
+    else:
+        H, st = mlstm_chunkwise__hip_xl_chunk(*leaves, **kw)
+    loss = (H.float() * cu(dH).float()).sum()
+    if c["dcl"]:
+        loss = loss + (st[0] * cu(dCl)).sum()
+    loss.backward()
     err = dict(H=rel_norm(H, fw["H"]), C=rel_to_scale(st[0], fw["C_last"]), dQ=rel_norm(leaves[0].grad, bw[0]),
                dK=rel_norm(leaves[1].grad, bw[1]), dV=rel_norm(leaves[2].grad, bw[2]),
                dI=rel_to_scale(leaves[3].grad, bw[3]), dF=rel_to_scale(leaves[4].grad, bw[4]))
