@@ -112,6 +112,24 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
                            int dtype_qkv, int dtype_gates, int gate, int normalize, int path, int state_stride,
                            void* stream);
 
+/*
+ * Allocation-free chunkwise forward (inference / prefill: nothing is kept for a backward pass).
+ * No counterpart in the reference.  For callers that cannot allocate device memory around the call -- code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc: same arguments and results as
+ * mlstm_hip_chunkwise_fw with keep_for_backward = 0, path = MLSTM_PATH_AUTO and state_stride = 0, but the workspace is
+ * a static device array of MLSTM_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
+ * ends) instead of a caller-provided buffer.  The call allocates and frees nothing.  Shapes whose workspace
+ * (mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0, MLSTM_PATH_AUTO, 0)) exceeds the static scratch are
+ * rejected.  All calls on one GPU share that GPU's scratch: calls that overlap in time on one GPU race.
+ */
+#define MLSTM_NOALLOC_SCRATCH_BYTES (64u << 20)
+int mlstm_hip_chunkwise_fw_noalloc(const void* q, const void* k, const void* v, const void* i, const void* f,
+                                   const float* c0, const float* n0, const float* m0,
+                                   void* H, float* n_out, float* m_out,
+                                   float* c_last, float* n_last, float* m_last,
+                                   int B, int NH, int S, int DHQK, int DHHV, float eps,
+                                   int dtype_qkv, int dtype_gates, int gate, int normalize, void* stream);
+
 /* Bytes of scratch the chunkwise backward needs in addition to the forward workspace. */
 size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int state_stride);
 
