@@ -210,11 +210,16 @@ def _chunk_gates(i, f, L: int, siging: bool):
 
 def chunkwise_fw(q, k, v, i, f, c_initial=None, n_initial=None, m_initial=None, chunk_size: int = 64,
                  eps: float = 1e-6, siging: bool = False, normalize: bool = True,
-                 return_all_states: bool = False):
+                 return_all_states: bool = False, return_bounds: bool = False):
     """Chunkwise-parallel forward.  Returns a dict with H (B,NH,S,DHV), n_out/m_out (B,NH,S) (the per-row
     denominator max(|den|, floor) *without* eps and the combined stabiliser), the last states and,
     on request, the per-chunk states C_all (B,NH,NC+1,DQK,DHV), n_all (B,NH,NC+1,DQK), m_all (B,NH,NC+1)
-    where index k holds the state *before* chunk k."""
+    where index k holds the state *before* chunk k.
+
+    ``return_bounds`` adds H_abs (B,NH,S,DHV): the sum of the MAGNITUDES of all products that enter an output element
+    in this chunk decomposition, (|qbar| |C_prev| + |Sbar| |V|) / (nmax + eps).  An implementation that rounds one
+    operand of every product to a p-bit significand deviates from the exact H by at most 2^-p H_abs (first order);
+    tests use it to bound the elements whose normaliser nearly cancels.  Not part of the reference's algorithm."""
     B, NH, S, DQK = q.shape
     DHV = v.shape[-1]
     L = chunk_size
@@ -228,6 +233,7 @@ def chunkwise_fw(q, k, v, i, f, c_initial=None, n_initial=None, m_initial=None, 
     m = torch.zeros(B, NH, dtype=dt, device=dev) if (m_initial is None or siging) else m_initial.to(dt).reshape(B, NH)
     causal = torch.ones(L, L, dtype=torch.bool, device=dev).tril()
     H = torch.empty(B, NH, S, DHV, dtype=dt, device=dev)
+    H_abs = torch.empty(B, NH, S, DHV, dtype=dt, device=dev) if return_bounds else None
     n_out = torch.ones(B, NH, S, dtype=dt, device=dev)
     m_out = torch.zeros(B, NH, S, dtype=dt, device=dev)
     C_all, n_all, m_all = [], [], []
@@ -248,13 +254,18 @@ def chunkwise_fw(q, k, v, i, f, c_initial=None, n_initial=None, m_initial=None, 
         bbar = torch.exp(bc + m[..., None] - m_comb)
         qbar = qc * (bbar * s)[..., None]
         num = qbar @ C + Sbar @ vc
+        num_abs = qbar.abs() @ C.abs() + Sbar.abs() @ vc.abs() if return_bounds else None
         if siging and not normalize:
             H[:, :, sl] = num
+            if return_bounds:
+                H_abs[:, :, sl] = num_abs
         else:
             den = (qbar * n[..., None, :]).sum(-1) + Sbar.sum(-1)
             floor = torch.ones_like(den) if siging else torch.exp(-m_comb)
             nmax = torch.maximum(den.abs(), floor)
             H[:, :, sl] = num / (nmax[..., None] + eps)
+            if return_bounds:
+                H_abs[:, :, sl] = num_abs / (nmax[..., None] + eps)
             n_out[:, :, sl] = nmax
         m_out[:, :, sl] = m_comb
         # ---- state update over this chunk (fw.py:88-121)
@@ -267,6 +278,8 @@ def chunkwise_fw(q, k, v, i, f, c_initial=None, n_initial=None, m_initial=None, 
             n = gbar[..., None] * n + kbar.sum(-2)
         m = m_next
     out = {"H": H, "n_out": n_out, "m_out": m_out, "C_last": C, "n_last": n, "m_last": m[..., None]}
+    if return_bounds:
+        out["H_abs"] = H_abs
     if return_all_states:
         C_all.append(C), n_all.append(n), m_all.append(m)
         out["C_all"] = torch.stack(C_all, 2)
@@ -276,11 +289,16 @@ def chunkwise_fw(q, k, v, i, f, c_initial=None, n_initial=None, m_initial=None, 
 
 
 def chunkwise_bw(q, k, v, i, f, dH, c_initial=None, n_initial=None, m_initial=None, dC_last=None,
-                 chunk_size: int = 64, eps: float = 1e-6, siging: bool = False, normalize: bool = True):
+                 chunk_size: int = 64, eps: float = 1e-6, siging: bool = False, normalize: bool = True,
+                 return_bounds: bool = False):
     """Chunkwise backward with the reference's convention: n_out and every stabiliser are constants
     (bw.py:44-46), dI = sum_d v*dV (bw.py:326, times sig(-i) for the sig gate), dF is the reverse
     cumulative sum over the WHOLE sequence of sum_d(q*dQ - k*dK) times sig(-f) (bw.py:320-323).
-    Returns dQ, dK, dV, dI, dF, dC_initial (None unless c_initial was given)."""
+    Returns dQ, dK, dV, dI, dF, dC_initial (None unless c_initial was given).
+
+    ``return_bounds`` appends a dict with dQ_abs, dK_abs, dV_abs: the sums of the magnitudes of all products entering
+    a gradient element in this chunk decomposition (the dC recurrence carried in magnitudes too, since an
+    implementation that rounds the operands of the dC update carries that error along).  See chunkwise_fw."""
     B, NH, S, DQK = q.shape
     DHV = v.shape[-1]
     L = chunk_size
@@ -298,6 +316,9 @@ def chunkwise_bw(q, k, v, i, f, dH, c_initial=None, n_initial=None, m_initial=No
     causal = torch.ones(L, L, dtype=torch.bool, device=dev).tril()
     dQ, dK, dV = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dC = torch.zeros_like(C_all[:, :, 0]) if dC_last is None else dC_last.to(q.dtype)
+    if return_bounds:
+        dQa, dKa, dVa = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dCa = dC.abs()
     for c_idx in range(NC - 1, -1, -1):
         sl = slice(c_idx * L, (c_idx + 1) * L)
         qc, kc, vc, dhc = q[:, :, sl], k[:, :, sl], v[:, :, sl], dHn[:, :, sl]
@@ -314,12 +335,19 @@ def chunkwise_bw(q, k, v, i, f, dH, c_initial=None, n_initial=None, m_initial=No
         dV[:, :, sl] = Sbar.transpose(-1, -2) @ dhc + (kc * abar) @ dC
         dK[:, :, sl] = (dS.transpose(-1, -2) @ qc) * s + (vc * abar) @ dC.transpose(-1, -2)
         dQ[:, :, sl] = (dS @ kc) * s + (dhc * bbar) @ (C_prev * s).transpose(-1, -2)
+        if return_bounds:
+            dVa[:, :, sl] = Sbar.abs().transpose(-1, -2) @ dhc.abs() + (kc.abs() * abar) @ dCa
+            dKa[:, :, sl] = (dS.abs().transpose(-1, -2) @ qc.abs()) * s + (vc.abs() * abar) @ dCa.transpose(-1, -2)
+            dQa[:, :, sl] = (dS.abs() @ kc.abs()) * s + (dhc.abs() * bbar) @ (C_prev.abs() * s).transpose(-1, -2)
+            dCa = gbar * dCa + (qc.abs() * bbar * s).transpose(-1, -2) @ dhc.abs()
         dC = gbar * dC + (qc * bbar * s).transpose(-1, -2) @ dhc
     acc = (q * dQ - k * dK).sum(-1)
     dF = acc.flip(-1).cumsum(-1).flip(-1) * torch.sigmoid(-f)
     dI = (v * dV).sum(-1)
     if siging:
         dI = dI * torch.sigmoid(-i)
+    if return_bounds:
+        return dQ, dK, dV, dI, dF, (dC if c_initial is not None else None), {"dQ_abs": dQa, "dK_abs": dKa, "dV_abs": dVa}
     return dQ, dK, dV, dI, dF, (dC if c_initial is not None else None)
 
 

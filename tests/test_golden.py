@@ -182,3 +182,86 @@ def test_chunkwise_fixture_hip(tag, sig):
     for name, t in (("dI", i), ("dF", f)):
         assert rel_to_scale(t.grad, z[f"{tag}_{name}"]) <= 5e-2, name
     assert rel_norm(c0.grad, z[f"{tag}_dC0"]) <= 5e-3
+
+
+# ------------------------------------------------------------------ reference-made vectors: sigmoid gate, decode step
+def _reference_siging_step(case):
+    """Outputs of the reference's own native_siging forward/backward and native decode step
+    (tests/golden/make_reference_vectors_siging_step.py)."""
+    z = np.load(os.path.join(GOLD, "reference_native_siging_step.npz"))
+    d = {k[len(case) + 1:]: torch.from_numpy(z[k]) for k in z.files if k.startswith(case + "_")}
+    return d, [int(x) for x in d.pop("meta")]
+
+
+@pytest.mark.parametrize("case", ["sigA", "sigB"])
+def test_oracle_matches_reference_siging_vectors(case):
+    """The oracle's quadratic AND chunkwise mLSTMsig (forward and hand-written backward) against the reference's
+    native_siging numbers (fp32-stored vectors: 1e-5)."""
+    z, (B, NH, S, DQK, DHV, normalize) = _reference_siging_step(case)
+    z = {k: v.double() for k, v in z.items()}
+    H, n = O.parallel_siging_fw(z["q"], z["k"], z["v"], z["i"], z["f"], normalize=bool(normalize))
+    torch.testing.assert_close(H, z["H"], rtol=1e-5, atol=1e-5)
+    if normalize:
+        torch.testing.assert_close(n, z["n"], rtol=1e-5, atol=1e-5)
+    grads = O.parallel_siging_bw(z["dH"], z["q"], z["k"], z["v"], z["i"], z["f"], n, normalize=bool(normalize))
+    for name, t in zip(["dQ", "dK", "dV", "dI", "dF"], grads):
+        torch.testing.assert_close(t, z[name], rtol=1e-5, atol=1e-5, msg=lambda s: f"{name}: {s}")
+    fw = O.chunkwise_fw(z["q"], z["k"], z["v"], z["i"], z["f"], chunk_size=32, siging=True, normalize=bool(normalize))
+    torch.testing.assert_close(fw["H"], z["H"], rtol=1e-5, atol=1e-5)
+    bw = O.chunkwise_bw(z["q"], z["k"], z["v"], z["i"], z["f"], z["dH"], chunk_size=32, siging=True, normalize=bool(normalize))
+    for name, t in zip(["dQ", "dK", "dV", "dI", "dF"], bw[:5]):
+        torch.testing.assert_close(t, z[name], rtol=2e-5, atol=2e-5, msg=lambda s: f"chunkwise {name}: {s}")
+
+
+@pytest.mark.parametrize("case", ["stepA", "stepB"])
+def test_oracle_matches_reference_step_vectors(case):
+    """The oracle's decode step, from random non-zero (C, n, m), against the reference's native step over a few
+    consecutive steps (fp32-stored vectors: 1e-5)."""
+    z, (B, NH, DQK, DHV, steps) = _reference_siging_step(case)
+    z = {k: v.double() for k, v in z.items()}
+    c, n, m = z["c0"], z["n0"], z["m0"]
+    for t in range(steps):
+        h, (c, n, m) = O.recurrent_step(z[f"q{t}"], z[f"k{t}"], z[f"v{t}"], z[f"i{t}"], z[f"f{t}"], c, n, m)
+        torch.testing.assert_close(h, z[f"h{t}"], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(c, z["c_last"], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(n, z["n_last"], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(m, z["m_last"], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["sigA", "sigB"])
+def test_hip_matches_reference_siging_vectors(case):
+    """The HIP mLSTMsig operator against the reference's native_siging numbers (bf16 operand bounds: outputs and
+    gradients 2e-2 on >= 99.9 % of the elements, 1e-2 of the scale, 5e-3 norm-wise; gate gradients 5e-2 of their scale)."""
+    from mlstm_kernels_amd.torch.chunkwise import mlstm_siging_chunkwise__hip_xl_chunk
+
+    z, (B, NH, S, DQK, DHV, normalize) = _reference_siging_step(case)
+    dev = "cuda"
+    q, k, v = (z[x].bfloat16().to(dev).requires_grad_(True) for x in "qkv")
+    i, f = z["i"].to(dev).requires_grad_(True), z["f"].to(dev).requires_grad_(True)
+    H = mlstm_siging_chunkwise__hip_xl_chunk(q, k, v, i, f, normalize=bool(normalize), chunk_size=128)
+    (H.float() * z["dH"].to(dev)).sum().backward()
+    for name, t in (("H", H), ("dQ", q.grad), ("dK", k.grad), ("dV", v.grad)):
+        assert allclose_frac(t, z[name], 2e-2, 2e-2) <= 1e-3, name
+        assert rel_to_scale(t, z[name]) <= 1e-2 and rel_norm(t, z[name]) <= 5e-3, name
+    for name, t in (("dI", i.grad), ("dF", f.grad)):
+        assert rel_to_scale(t, z[name]) <= 5e-2, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["stepA", "stepB"])
+def test_hip_step_matches_reference_step_vectors(case):
+    """The HIP decode step, state carried over a few consecutive steps, against the reference's native step: fp32
+    states 1e-5 relative, h within bf16 rounding of the output (5e-3 of the scale)."""
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip
+
+    z, (B, NH, DQK, DHV, steps) = _reference_siging_step(case)
+    dev = "cuda"
+    c, n, m = z["c0"].to(dev), z["n0"].to(dev), z["m0"].to(dev)
+    for t in range(steps):
+        h, (c, n, m) = mlstm_recurrent_step__hip(z[f"q{t}"].bfloat16().to(dev), z[f"k{t}"].bfloat16().to(dev),
+                                                 z[f"v{t}"].bfloat16().to(dev), z[f"i{t}"].to(dev), z[f"f{t}"].to(dev), c, n, m)
+        assert rel_to_scale(h, z[f"h{t}"]) <= 5e-3, f"h at step {t}"
+    assert_state_close(c, z["c_last"], 1e-5, "C")
+    assert_state_close(n, z["n_last"], 1e-5, "n")
+    assert (m.cpu() - z["m_last"]).abs().max() <= 1e-5

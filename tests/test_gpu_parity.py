@@ -3,9 +3,13 @@ oracle on the same seeded, bf16-rounded inputs.
 
 Stated tolerances (bf16 inputs, fp32 states):
   * H, dQ, dK, dV: |x - ref| <= 2e-2 + 2e-2 |ref| element-wise.  The matrix kernels feed bf16-rounded operands
-    (gated scores, chunk states) to the matrix cores, so rows whose normaliser nearly cancels amplify a 2^-9
-    operand rounding beyond that bound on a few elements in 10^4; the tests therefore require the bound on
-    >= 99.9 % of the elements AND max|x - ref| <= 1e-2 max|ref| AND ||x - ref|| <= 5e-3 ||ref||.
+    (gated scores, chunk states) to the matrix cores: one operand of every product carries a relative rounding error
+    of up to 2^-8 (8-bit significand).  On rows whose normaliser nearly cancels the products are large against their
+    sum and that rounding exceeds the bound on a few elements in 10^4.  The tests therefore require
+      - the bound on >= 99.9 % of the elements, max|x - ref| <= 1e-2 max|ref|, ||x - ref|| <= 5e-3 ||ref||, and
+      - on EVERY element |x - ref| <= 2e-2 + 2e-2 |ref| + 1.25 * 2^-8 * A, where A is the sum of the magnitudes of all
+        products entering that element (computed by the oracle in the same chunk decomposition): the first-order
+        worst case of the operand roundings.  The count of offenders and the worst one are printed per tensor.
   * final C / n / m states: 1e-3 relative (max error over tensor scale, and norm-wise).
   * dI, dF: 5e-2 of the tensor scale (sums over the head dimension / the whole sequence of differences of
     bf16-rounded products; the reference's own tests allow atol 0.4 there).
@@ -23,11 +27,12 @@ DEV = "cuda"
 _VARIANT = {"kernel_path": "auto", "chunk_size_intra": None}
 
 
-@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "fused-2"])
+@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "fused-1"])
 def kernel_variant(request):
     """Every test runs once per kernel variant of the chunkwise passes: the split path (state scan + chunk-parallel
     kernels) with a chunk state kept every 1, 2 or 4 chunks, and the fused path (sequential kernels with a
-    register-resident state; head dimensions it does not support are skipped)."""
+    register-resident state; head dimensions it does not support are skipped; stride 1, so that all its kernels group
+    the products the same way -- the fused path with other strides is part of the randomised sweep)."""
     path, stride = request.param.split("-")
     _VARIANT.update(kernel_path=path, chunk_size_intra=128 * int(stride))
     yield request.param
@@ -71,12 +76,42 @@ def report_offenders(x, ref, name, rtol=2e-2, atol=2e-2):
     return n_bad / ratio.numel(), worst
 
 
-def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3, worst_tol=12.0):
+_U_BF16 = 2.0 ** -8   # unit roundoff of an 8-bit significand
+
+
+def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3, worst_tol=12.0, abs_sum=None):
+    """`abs_sum` (same shape as ref): magnitude sum of the products entering each element; when given, every element
+    must lie within the 2e-2/2e-2 bound widened by the worst case of one operand rounding per product."""
     bad, worst = report_offenders(x, ref, name)
     e1, e2 = rel_to_scale(x, ref), rel_norm(x, ref)
     assert bad <= frac and worst <= worst_tol and e1 <= scale_tol and e2 <= norm_tol, (
         f"{name}: {bad:.2e} of elements outside 2e-2/2e-2 (worst {worst:.2f} x the bound), max err / scale {e1:.2e}, "
         f"norm err {e2:.2e}")
+    if abs_sum is not None:
+        x64, r64 = x.detach().double().cpu(), ref.detach().double().cpu()
+        slack = (x64 - r64).abs() - (2e-2 + 2e-2 * r64.abs() + 1.25 * _U_BF16 * abs_sum.double().cpu())
+        n_out = int((slack > 0).sum())
+        assert n_out == 0, (f"{name}: {n_out} elements exceed the 2e-2/2e-2 bound by more than the operand-rounding "
+                            f"worst case (largest excess {float(slack.max()):.3e})")
+
+
+def bound_chunk(S):
+    """Chunk length at which the oracle's magnitude sums describe the running kernel variant: the kernel groups the
+    products exactly like the chunkwise formulation with chunks of 128 positions times the state stride (one chunk if
+    the sequence is shorter).  None when the sequence length does not fit that decomposition (ragged lengths): such
+    tests check the other bounds only."""
+    L = 128 * ((_VARIANT["chunk_size_intra"] or 256) // 128)
+    if S <= L:
+        return S
+    return L if S % L == 0 else None
+
+
+def oracle_chunk(S):
+    """(chunk length for the oracle, whether its magnitude sums apply to the running kernel variant)."""
+    L = bound_chunk(S)
+    if L is not None:
+        return L, True
+    return next(c for c in (128, 64, 32, 16, 8, 4, 2, 1) if S % c == 0), False
 
 
 def d64(t):
@@ -210,12 +245,13 @@ def test_decode_steps_in_hip_graph():
 def test_chunkwise_forward_exp(cfg):
     exp_op, *_ = _ops()
     q, k, v, i, f = make_qkvif(cfg["B"], cfg["NH"], cfg["S"], cfg["DQK"], cfg["DHV"], cfg["seed"])
-    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=min(cfg["L"], 64))
+    Lo, bounded = oracle_chunk(cfg["S"])
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=Lo, return_bounds=True)
     args = [t.to(DEV) for t in (q.to(cfg["dtype"]), k.to(cfg["dtype"]), v.to(cfg["dtype"]), i, f)]
     H, (C, n, m) = exp_op(*args, return_last_states=True, chunk_size=cfg["L"])
     assert H.dtype == cfg["dtype"] and H.shape == v.shape and C.dtype == torch.float32
     assert m.shape == (cfg["B"], cfg["NH"], 1)
-    check_matrix(H, ref["H"], "H")
+    check_matrix(H, ref["H"], "H", abs_sum=ref["H_abs"] if bounded else None)
     assert_state_close(C, ref["C_last"], 1e-3, "C_last")
     assert_state_close(n, ref["n_last"], 1e-3, "n_last")
     assert (d64(m) - ref["m_last"]).abs().max() <= 1e-3
@@ -228,9 +264,10 @@ def test_chunkwise_forward_exp(cfg):
 def test_chunkwise_forward_gate_regimes(f_offset, DQK):
     exp_op, *_ = _ops()
     q, k, v, i, f = make_qkvif(1, 2, 384, DQK, 128, seed=7, f_offset=f_offset)
-    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=64)
+    Lo, bounded = oracle_chunk(384)
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=Lo, return_bounds=True)
     H, (C, n, m) = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
-    check_matrix(H, ref["H"], "H", frac=2e-3)
+    check_matrix(H, ref["H"], "H", frac=2e-3, abs_sum=ref["H_abs"] if bounded else None)
     assert_state_close(C, ref["C_last"], 1e-3, "C_last")
     assert (d64(m) - ref["m_last"]).abs().max() <= 1e-3
 
@@ -271,19 +308,21 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     loss.backward()
     # oracle on a subset of (batch, head) pairs: every pair is independent
     pairs = pairs or [(b, h) for b in range(B) for h in range(NH)]
-    Lo = next(c for c in (128, 64, 32, 16) if S % c == 0)   # the oracle's chunk length (results do not depend on it)
+    Lo, bounded = oracle_chunk(S)   # the oracle's chunk length (its results do not depend on it, its magnitude sums do)
     for (b, h) in pairs:
         sl = lambda t: None if t is None else d64(t[b:b + 1, h:h + 1])
-        fw = O.chunkwise_fw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(c0), sl(n0), sl(m0), chunk_size=Lo, siging=siging, normalize=normalize)
-        bw = O.chunkwise_bw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(dH), sl(c0), sl(n0), sl(m0), sl(dCl), chunk_size=Lo, siging=siging, normalize=normalize)
+        fw = O.chunkwise_fw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(c0), sl(n0), sl(m0), chunk_size=Lo, siging=siging,
+                            normalize=normalize, return_bounds=True)
+        bw = O.chunkwise_bw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(dH), sl(c0), sl(n0), sl(m0), sl(dCl), chunk_size=Lo,
+                            siging=siging, normalize=normalize, return_bounds=True)
         tag = f"(b={b},h={h})"
-        check_matrix(H[b:b + 1, h:h + 1], fw["H"], "H" + tag)
+        check_matrix(H[b:b + 1, h:h + 1], fw["H"], "H" + tag, abs_sum=fw["H_abs"] if bounded else None)
         assert_state_close(st[0][b:b + 1, h:h + 1], fw["C_last"], 1e-3, "C_last" + tag)
         assert_state_close(st[1][b:b + 1, h:h + 1], fw["n_last"], 1e-3, "n_last" + tag)
         if not siging:
             assert (d64(st[2][b:b + 1, h:h + 1]) - fw["m_last"]).abs().max() <= 1e-3
         for name, leaf, r in zip(["dQ", "dK", "dV"], leaves[:3], bw[:3]):
-            check_matrix(leaf.grad[b:b + 1, h:h + 1], r, name + tag)
+            check_matrix(leaf.grad[b:b + 1, h:h + 1], r, name + tag, abs_sum=bw[6][name + "_abs"] if bounded else None)
         for name, leaf, r in zip(["dI", "dF"], leaves[3:], bw[3:5]):
             e = rel_to_scale(leaf.grad[b:b + 1, h:h + 1], r)
             assert e <= 5e-2, f"{name}{tag}: max err / scale {e:.2e}"
@@ -313,12 +352,12 @@ def test_chunkwise_fwbw_small(kw):
 def test_chunkwise_fwbw_xlstm7b_shape_exp(B, S):
     """BASELINE config 3: NH=8, DHQK=256, DHHV=512, B*S = 65536, upstream dH ~ N(0,1).  The whole tensor runs on
     the GPU; two (batch, head) pairs are checked against the fp64 oracle over the full sequence."""
-    _fwbw_case(B, 8, S, 256, 512, seed=0, pairs=[(0, 0), (B - 1, 5)])
+    _fwbw_case(B, 8, S, 256, 512, seed=0, pairs=[(0, 0), (B - 1, 7)])   # first and last workgroups of every launch
 
 
 def test_chunkwise_fwbw_xlstm7b_shape_sig():
     """BASELINE config 4: mLSTMsig, B=4, S=16384, non-zero initial C ~ N(0,0.1), n ~ N(0,0.1), m = 0."""
-    _fwbw_case(4, 8, 16384, 256, 512, siging=True, init=True, seed=0, pairs=[(1, 3), (3, 7)])
+    _fwbw_case(4, 8, 16384, 256, 512, siging=True, init=True, seed=0, pairs=[(1, 4), (2, 3)])   # middle of the grid
 
 
 # ------------------------------------------------------------------------------------------ size-independent properties
