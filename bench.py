@@ -4,25 +4,36 @@
 A "step" is one TFLA forward + backward pass (mLSTMexp, upstream dH ~ N(0,1)) over the xLSTM-7B layer shape
 B=4, S=16384, NH=8, DHQK=256, DHHV=512, chunk_size=128, bf16 inputs / fp32 states, synthetic N(0,1) data resident
 in HBM before the timed region.  `value` is algorithmic TFLOP/s: 0.9964 TFLOP per step (matmul flops only,
-causal work counted once, no recomputation) divided by the measured time per step.  The same run also times the
-fused decode step (B=256, 128 consecutive steps after a chunkwise prefill) and reports it as algorithmic GB/s.
+causal work counted once, no recomputation) divided by the time per step.
 
-Extra objects on the JSON line:
-  roofline      -- the chunkwise kernel with the largest share of the step (MFMA bound): algorithmic flops of one
-                   launch / its average duration, measured with HIP events the library records around every
-                   kernel launch on the launch stream during the timed region.
-  kernels       -- the same figure for every kernel of the step.
-  decode_step   -- ms per step, algorithmic GB/s and its own HBM roofline object.
-  cpu_baseline  -- the fp32 PyTorch oracle (a restatement of the reference's native chunkwise forward + custom
-                   backward) timed on this box's host cores on a bounded sample of the same workload.
+Timing protocol (the reference's, mlstm_kernels/utils/benchmark/runtime.py:30-170): W untimed warm-up steps, then
+exactly K timed steps; before every step a 512 MB buffer is zeroed to flush the L2 and the 256 MB memory-side cache,
+gradients are reset, and the step is bracketed by a pair of HIP events on the launch stream; `ms_per_step` is the
+MEDIAN of the K event times (the mean and the wall clock over the whole loop, flushes included, are reported next to
+it).  Per-kernel durations come from a SEPARATE untimed pass over the same workload, in which the library records a
+pair of HIP events around every kernel launch (mlstm_hip_profile_enable).
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+Objects on the JSON line besides the contract's keys:
+  roofline      -- the chunkwise kernel with the largest share of the step against the bf16 MFMA peak: algorithmic
+                   flops of one launch / its average duration; `traffic` = measured HBM bytes per launch, parsed from
+                   the rocprofv3 counter summary under profiles/ (null when that file has no row for the kernel).
+  roofline_hbm  -- the same kernel against the HBM peak (algorithmic bytes per launch).
+  kernels       -- average duration, algorithmic TFLOP/s and GB/s of every kernel of the step.
+  decode_step   -- fused decode step at B=256 after a chunkwise prefill of 2048 positions: ms per step, algorithmic
+                   GB/s, its own HBM roofline; B=64 and B=16 (whose state fits the memory-side cache: "bound": "mall").
+  extra         -- the other BASELINE configurations, same protocol: B=16/S=4096 and B=64/S=1024 (fwd+bwd), the
+                   sigmoid gate with a non-zero initial state at B=4/S=16384, and forward-only at B=4/S=16384.
+  cpu_baseline  -- the fp32 PyTorch oracle (restatement of the reference's native chunkwise forward + custom backward)
+                   timed on this box's host cores on the same workload, plus the oracle's decode step.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra]
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -34,52 +45,74 @@ B, S, NH, DHQK, DHHV, CHUNK = 4, 16384, 8, 256, 512, 128
 TOKEN_HEADS = B * S * NH
 FLOPS_PER_TOKEN_HEAD = {
     # forward: 4*dqk*dhv + L*(dqk+dhv) = 622592
-    "scan_fw": 2 * DHQK * DHHV,                       # K^T (a.V)
-    "par_h": 2 * DHQK * DHHV + CHUNK * (DHQK + DHHV),  # Q C_prev, causal Q K^T and Sbar V
+    "scan_fw": 2 * DHQK * DHHV,                         # K^T (a.V)
+    "par_h": 2 * DHQK * DHHV + CHUNK * (DHQK + DHHV),   # Q C_prev, causal Q K^T and Sbar V
     # backward: 8*dqk*dhv + L*(3*dqk + 2*dhv) = 1277952
-    "scan_bw": 2 * DHQK * DHHV,                       # Q^T dH
+    "scan_bw": 2 * DHQK * DHHV,                         # Q^T dH
     "par_dv": 2 * DHQK * DHHV + CHUNK * (DHQK + DHHV),  # K dC, causal Q K^T and Sbar^T dH
-    "par_dq": 2 * DHQK * DHHV + CHUNK * (DHHV + DHQK),  # dH C^T, causal dH V^T and dS K
-    "par_dk": 2 * DHQK * DHHV + CHUNK * DHQK,           # V dC^T, causal dS^T Q
+    # dQ and dK run as one launch: dH C^T, causal dH V^T and dS K; V dC^T, causal dS^T Q
+    "par_dqdk": 2 * DHQK * DHHV + CHUNK * (DHHV + DHQK) + 2 * DHQK * DHHV + CHUNK * DHQK,
 }
 # the fused sequential kernels do the work of a scan plus the chunk-parallel kernel that follows it
 FLOPS_PER_TOKEN_HEAD["fused_fw"] = FLOPS_PER_TOKEN_HEAD["scan_fw"] + FLOPS_PER_TOKEN_HEAD["par_h"]
 FLOPS_PER_TOKEN_HEAD["fused_dv"] = FLOPS_PER_TOKEN_HEAD["scan_bw"] + FLOPS_PER_TOKEN_HEAD["par_dv"]
-# dQ and dK run as one launch
-FLOPS_PER_TOKEN_HEAD["par_dqdk"] = FLOPS_PER_TOKEN_HEAD.pop("par_dq") + FLOPS_PER_TOKEN_HEAD.pop("par_dk")
 FLOPS_FW = 4 * DHQK * DHHV + CHUNK * (DHQK + DHHV)
 FLOPS_BW = 8 * DHQK * DHHV + CHUNK * (3 * DHQK + 2 * DHHV)
 assert sum(FLOPS_PER_TOKEN_HEAD[n] for n in ("fused_fw", "fused_dv", "par_dqdk")) == FLOPS_FW + FLOPS_BW
-# algorithmic HBM bytes per launch at this workload: every operand once (bf16 q/k 268 MB, v/dH/H 537 MB, bf16 chunk
-# states 1074 MB per tensor)
-_QB, _VB = B * NH * S * DHQK * 2, B * NH * S * DHHV * 2
-_SB = B * NH * (S // CHUNK) * DHQK * DHHV * 2
-ALG_BYTES = {
-    "scan_fw": _QB + _VB + _SB, "par_h": 2 * _QB + 2 * _VB + _SB,
-    "scan_bw": _QB + _VB + _SB, "par_dv": 2 * _QB + 2 * _VB + _SB,
-    "par_dqdk": 4 * _QB + 2 * _VB + 2 * _SB,   # Q, K, V, dH once for both gradients; C and dC states; dQ, dK out
-}
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload (calibrated against a
-# copy kernel of known size; summary in profiles/tfla_fwbw_B4_S16384__step_B256__pmc_hbm_traffic.md)
-MEASURED_HBM_BYTES = {
-    "scan_fw": 2122e6, "par_h": 2763e6, "scan_bw": 1883e6, "par_dv": 2890e6, "par_dqdk": 4319e6,
-    "step": 2163e6,
-}
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+FLUSH_BYTES = 512 << 20     # twice the memory-side cache
 # decode step: bytes per (batch, head): C and n read+write fp32, m read+write, q,k,v in, h out (bf16), i,f
 STEP_BYTES_PER_BH = 2 * DHQK * DHHV * 4 + 2 * DHQK * 4 + 2 * 4 + (2 * DHQK + DHHV) * 2 + DHHV * 2 + 2 * 2
 DECODE_B, DECODE_PREFILL, DECODE_STEPS, DECODE_WARMUP = 256, 2048, 128, 10
+MALL_BYTES = 256 << 20
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "tfla_fwbw_B4_S16384__pmc_hbm_traffic.md")
+
+
+def algorithmic_bytes(stride: int) -> dict:
+    """HBM bytes per launch if every operand moved once: bf16 q/k 268 MB each, v/dH/H/dV 537 MB each, bf16 chunk states
+    (one per `stride` chunks of 128 positions) 1074 MB / stride per tensor."""
+    qb, vb = B * NH * S * DHQK * 2, B * NH * S * DHHV * 2
+    sb = B * NH * -(-(S // CHUNK) // stride) * DHQK * DHHV * 2
+    return {
+        "scan_fw": qb + vb + sb, "par_h": 2 * qb + 2 * vb + sb,
+        "scan_bw": qb + vb + sb, "par_dv": 2 * qb + 2 * vb + sb,
+        "par_dqdk": 4 * qb + 2 * vb + 2 * sb,   # Q, K, V, dH once for both gradients; C and dC states; dQ, dK out
+    }
+
+
+def measured_traffic() -> dict:
+    """{kernel: HBM bytes per launch} parsed from the rocprofv3 FETCH_SIZE / WRITE_SIZE summary under profiles/
+    (table rows `| kernel | fetched MB | written MB | total MB |`); empty when the file is absent."""
+    out = {}
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return out
+    for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
+        out[m.group(1)] = float(m.group(4)) * 1e6
+    return out
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def cpu_baseline(torch):
-    """fp32 oracle forward+backward on a bounded sample: 8 of the 32 (batch, head) pairs, full S."""
+    """fp32 oracle on the host cores this process may use (the thread count the environment sets for one GPU's share of
+    the box): chunkwise forward+backward on the whole workload (all 32 (batch, head) pairs at S=16384), and the decode
+    step at B=16."""
     import oracle as O
 
-    threads = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
+    threads = torch.get_num_threads()
     g = torch.Generator().manual_seed(0)
-    nh_s = 32  # the whole workload: every (batch, head) pair is independent, so one "batch" of 32 heads
+    nh_s = B * NH  # every (batch, head) pair is independent, so one "batch" of 32 heads
     q = torch.randn(1, nh_s, S, DHQK, generator=g).bfloat16().float()
     k = torch.randn(1, nh_s, S, DHQK, generator=g).bfloat16().float()
     v = torch.randn(1, nh_s, S, DHHV, generator=g).bfloat16().float()
@@ -88,15 +121,32 @@ def cpu_baseline(torch):
     f = 3 + torch.randn(1, nh_s, S, generator=g)
     O.chunkwise_bw(q[:, :1, :1024], k[:, :1, :1024], v[:, :1, :1024], i[:, :1, :1024], f[:, :1, :1024], dH[:, :1, :1024], chunk_size=CHUNK)
     times = []
-    for _ in range(9):
+    for _ in range(5):
         t0 = time.perf_counter()
         O.chunkwise_bw(q, k, v, i, f, dH, chunk_size=CHUNK)   # runs the forward (all states) and the backward
         times.append(time.perf_counter() - t0)
     t = sorted(times)[len(times) // 2]
     flops = (FLOPS_FW + FLOPS_BW) * nh_s * S
+    del q, k, v, dH, i, f
+    # decode step: python loop of the oracle step, fp32 state, B=16
+    Bd, nsteps = 16, 12
+    c, n, m = torch.randn(Bd, NH, DHQK, DHHV, generator=g), torch.randn(Bd, NH, DHQK, generator=g), torch.randn(Bd, NH, 1, generator=g)
+    toks = [(torch.randn(Bd, NH, DHQK, generator=g), torch.randn(Bd, NH, DHQK, generator=g), torch.randn(Bd, NH, DHHV, generator=g),
+             torch.randn(Bd, NH, 1, generator=g), 3 + torch.randn(Bd, NH, 1, generator=g)) for _ in range(nsteps + 2)]
+    st = []
+    for idx, tok in enumerate(toks):
+        t0 = time.perf_counter()
+        _, (c, n, m) = O.recurrent_step(*tok, c, n, m)
+        if idx >= 2:
+            st.append(time.perf_counter() - t0)
+    ts = sorted(st)[len(st) // 2]
     return {
         "value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": f"fp32 oracle fwd+bwd on all {B * NH} (batch,head) pairs at S={S}: {t:.2f} s per pass, median of 9 after a warm-up",
+        "cpu_model": cpu_model(), "host_logical_cpus": os.cpu_count(),
+        "sample": f"fp32 oracle fwd+bwd on all {B * NH} (batch,head) pairs at S={S}: {t:.2f} s per pass, median of 5 after a "
+                  f"warm-up; {threads} threads = this process's share of the host",
+        "decode_step": {"value": round(STEP_BYTES_PER_BH * Bd * NH / ts / 1e9, 2), "unit": "GB/s", "ms_per_step": round(ts * 1e3, 3),
+                        "sample": f"fp32 oracle step at B={Bd}, NH={NH}: median of {nsteps} consecutive steps after 2 warm-up steps"},
     }
 
 
@@ -106,6 +156,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configurations and the small decode batches")
+    ap.add_argument("--state-stride", type=int, default=0, help="chunk states kept every n-th chunk (0 = library default)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures the hot path on ONE GPU; --gpus > 1 is not supported "
@@ -115,7 +167,7 @@ def main():
     import torch
 
     from mlstm_kernels_amd import _lib
-    from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk
+    from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk, mlstm_siging_chunkwise__hip_xl_chunk
     from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw
 
     _lib.get_lib()  # fail loudly if the HIP library is missing
@@ -126,55 +178,110 @@ def main():
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(0)
     rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
-    q = rn(B, NH, S, DHQK).bfloat16().requires_grad_(True)
-    k = rn(B, NH, S, DHQK).bfloat16().requires_grad_(True)
-    v = rn(B, NH, S, DHHV).bfloat16().requires_grad_(True)
-    i = rn(B, NH, S).requires_grad_(True)
-    f = (3 + rn(B, NH, S)).requires_grad_(True)
-    dH = rn(B, NH, S, DHHV).bfloat16()
+    flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
+    intra = {} if args.state_stride == 0 else {"chunk_size_intra": CHUNK * args.state_stride}
+    stride = args.state_stride or _lib.default_state_stride(B, NH, S, DHQK, DHHV)
 
-    def step():
-        for t in (q, k, v, i, f):
-            t.grad = None
-        H = mlstm_chunkwise__hip_xl_chunk(q, k, v, i, f, chunk_size=CHUNK, autocast_kernel_dtype=torch.bfloat16)
-        H.backward(dH)
+    def run_config(Bc, Sc, steps, warmup, sig=False, init=False, backward=True, profile_steps=3):
+        """Times `steps` passes of one configuration (median of per-step HIP-event times, caches flushed before every
+        step), then profiles `profile_steps` further passes kernel by kernel."""
+        q = rn(Bc, NH, Sc, DHQK).bfloat16().requires_grad_(backward)
+        k = rn(Bc, NH, Sc, DHQK).bfloat16().requires_grad_(backward)
+        v = rn(Bc, NH, Sc, DHHV).bfloat16().requires_grad_(backward)
+        i = rn(Bc, NH, Sc).requires_grad_(backward)
+        f = (3 + rn(Bc, NH, Sc)).requires_grad_(backward)
+        dH = rn(Bc, NH, Sc, DHHV).bfloat16()
+        kw = dict(chunk_size=CHUNK, autocast_kernel_dtype=torch.bfloat16, **intra)
+        if init:
+            kw.update(c_initial=0.1 * rn(Bc, NH, DHQK, DHHV), n_initial=0.1 * rn(Bc, NH, DHQK),
+                      m_initial=torch.zeros(Bc, NH, 1, device=dev))
+        op = mlstm_siging_chunkwise__hip_xl_chunk if sig else mlstm_chunkwise__hip_xl_chunk
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    _lib.profile_enable(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    _lib.profile_enable(False)
-    kern = _lib.profile_read()
-    ms_per_step = elapsed / args.steps * 1e3
+        def step():
+            if backward:
+                op(q, k, v, i, f, **kw).backward(dH)
+            else:
+                with torch.no_grad():
+                    op(q, k, v, i, f, **kw)
+
+        def prepare():
+            for t in (q, k, v, i, f):
+                t.grad = None
+            flush.zero_()
+
+        for _ in range(warmup):
+            prepare()
+            step()
+        torch.cuda.synchronize()
+        events = []
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            prepare()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            step()
+            e1.record()
+            events.append((e0, e1))
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        times = sorted(a.elapsed_time(b) for a, b in events)
+        median, mean = times[len(times) // 2], sum(times) / len(times)
+        # separate untimed pass: per-kernel durations
+        _lib.profile_read()
+        _lib.profile_enable(True)
+        for _ in range(profile_steps):
+            prepare()
+            step()
+        torch.cuda.synchronize()
+        _lib.profile_enable(False)
+        kern = {name: (ms / max(cnt, 1), cnt) for name, (ms, cnt) in _lib.profile_read().items()}
+        return {"median_ms": median, "mean_ms": mean, "min_ms": times[0], "wall_ms_incl_flush": wall / steps * 1e3, "kernels": kern}
+
+    def kernel_table(kern, token_heads, alg_bytes=None):
+        table = {}
+        for name, (avg, cnt) in kern.items():
+            entry = {"avg_ms": round(avg, 4), "launches": cnt}
+            if name in FLOPS_PER_TOKEN_HEAD:
+                entry["alg_tflops"] = round(FLOPS_PER_TOKEN_HEAD[name] * token_heads / (avg * 1e-3) / 1e12, 2)
+            if alg_bytes and name in alg_bytes:
+                entry["alg_gbs"] = round(alg_bytes[name] / (avg * 1e-3) / 1e9, 1)
+            table[name] = entry
+        return table
+
+    # ---- headline: mLSTMexp fwd+bwd, B=4, S=16384
+    head = run_config(B, S, args.steps, args.warmup, profile_steps=5)
+    ms_per_step = head["median_ms"]
     tflops = (FLOPS_FW + FLOPS_BW) * TOKEN_HEADS / (ms_per_step * 1e-3) / 1e12
-
-    kernels = {}
-    for name, (ms, cnt) in kern.items():
-        avg = ms / max(cnt, 1)
-        entry = {"avg_ms": round(avg, 4), "launches": cnt}
-        if name in FLOPS_PER_TOKEN_HEAD:
-            entry["alg_tflops"] = round(FLOPS_PER_TOKEN_HEAD[name] * TOKEN_HEADS / (avg * 1e-3) / 1e12, 2)
-        kernels[name] = entry
+    alg_bytes = algorithmic_bytes(stride)
+    kernels = kernel_table(head["kernels"], TOKEN_HEADS, alg_bytes)
+    traffic = measured_traffic()
     dom = max((n for n in kernels if n in FLOPS_PER_TOKEN_HEAD), key=lambda n: kernels[n]["avg_ms"])
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["alg_tflops"], "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s", "frac": round(kernels[dom]["alg_tflops"] / PEAK_BF16_TFLOPS, 4),
-        "traffic": MEASURED_HBM_BYTES.get(dom), "avg_launch_ms": kernels[dom]["avg_ms"],
+        "traffic": traffic.get(dom), "avg_launch_ms": kernels[dom]["avg_ms"],
     }
-    # the same kernel against the HBM roofline (at 65 flop per byte of materialised-state traffic the step is
-    # bandwidth-bound; both fractions are reported)
-    gbs = ALG_BYTES[dom] / (kernels[dom]["avg_ms"] * 1e-3) / 1e9
-    roofline_hbm = {"bound": "hbm", "kernel": dom, "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_HBM_BYTES.get(dom)}
+    # the same kernel against the HBM roofline (with materialised chunk states the step is bandwidth-bound; both
+    # fractions are reported)
+    roofline_hbm = {"bound": "hbm", "kernel": dom, "achieved": kernels[dom]["alg_gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(kernels[dom]["alg_gbs"] / PEAK_HBM_GBS, 4), "traffic": traffic.get(dom)}
     for name, entry in kernels.items():
-        if name in ALG_BYTES:
-            entry["alg_gbs"] = round(ALG_BYTES[name] / (entry["avg_ms"] * 1e-3) / 1e9, 1)
-    del q, k, v, i, f, dH
+        if name in traffic:
+            entry["hbm_bytes_measured"] = traffic[name]
+
+    extra = {}
+    if not args.no_extra:
+        n_extra = max(5, args.steps // 2)
+        for tag, cfg in (("exp_fwbw_B16_S4096", dict(Bc=16, Sc=4096)), ("exp_fwbw_B64_S1024", dict(Bc=64, Sc=1024)),
+                         ("sig_fwbw_B4_S16384_init", dict(Bc=4, Sc=16384, sig=True, init=True)),
+                         ("exp_fw_B4_S16384", dict(Bc=4, Sc=16384, backward=False))):
+            r = run_config(steps=n_extra, warmup=2, **cfg)
+            fl = (FLOPS_FW + (FLOPS_BW if cfg.get("backward", True) else 0)) * TOKEN_HEADS
+            extra[tag] = {"ms_per_step": round(r["median_ms"], 4), "steps": n_extra,
+                          "value": round(fl / (r["median_ms"] * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                          "kernels": kernel_table(r["kernels"], TOKEN_HEADS)}
+            torch.cuda.empty_cache()
+    del flush
     torch.cuda.empty_cache()
 
     # ---- decode step: chunkwise prefill, then consecutive in-place steps (state carried, n/m ping-pong)
@@ -189,6 +296,8 @@ def main():
         is_, fs = rn(total, Bd, NH, 1), 3 + rn(total, Bd, NH, 1)
         n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
         step_bytes = STEP_BYTES_PER_BH * Bd * NH
+        # a state that fits the memory-side cache is served from it step after step: not an HBM figure
+        bound = "hbm" if c.numel() * 4 > MALL_BYTES else "mall"
         if graph:
             # two steps (n/m ping-pong) per graph, tokens in static buffers refreshed by device-side copies
             sq, sk, sv = qs[:2].clone(), ks[:2].clone(), vs[:2].clone()
@@ -212,7 +321,7 @@ def main():
             torch.cuda.synchronize()
             dec_ms = (time.perf_counter() - t_dec) / DECODE_STEPS * 1e3
             return {"batch": Bd, "mode": "hip graph (2 steps per replay, incl. token copies)", "ms_per_step": round(dec_ms, 4),
-                    "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s"}
+                    "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "bound": bound}
         _lib.profile_read()
         t_dec = 0.0
         for t in range(total):
@@ -230,15 +339,16 @@ def main():
         step_kernel_ms = st_ms / max(st_cnt, 1)
         return {
             "batch": Bd, "mode": "eager", "steps": DECODE_STEPS, "ms_per_step": round(dec_ms, 4), "kernel_ms": round(step_kernel_ms, 4),
-            "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
-            "roofline": {"bound": "hbm", "kernel": "step", "achieved": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9, 1),
+            "value": round(step_bytes / (dec_ms * 1e-3) / 1e9, 1), "unit": "GB/s", "bound": bound,
+            "roofline": {"bound": bound, "kernel": "step", "achieved": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(step_bytes / (step_kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                         "traffic": MEASURED_HBM_BYTES["step"] if Bd == DECODE_B else None},
+                         "traffic": traffic.get("step") if Bd == DECODE_B else None},
         }
 
     decode = bench_decode(DECODE_B, graph=False)
-    decode["other_batches"] = [bench_decode(b, graph=g_) for b in (64, 16) for g_ in (False, True)]
+    if not args.no_extra:
+        decode["other_batches"] = [bench_decode(b, graph=g_) for b in (64, 16) for g_ in (False, True)]
     torch.cuda.empty_cache()
 
     out = {
@@ -247,8 +357,11 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "mLSTMexp TFLA fwd+bwd, B=4 S=16384 NH=8 DHQK=256 DHHV=512 chunk=128 (BASELINE configs[2]); "
-                               "decode step B=256 (configs[4])"},
-        "roofline": roofline, "roofline_hbm": roofline_hbm, "kernels": kernels, "decode_step": decode,
+                               "decode step B=256 (configs[4])", "state_stride": stride},
+        "timing": {"protocol": "median of per-step HIP-event times, 512 MB cache flush and gradient reset before every step",
+                   "mean_ms": round(head["mean_ms"], 4), "min_ms": round(head["min_ms"], 4),
+                   "wall_ms_per_step_incl_flush": round(head["wall_ms_incl_flush"], 4)},
+        "roofline": roofline, "roofline_hbm": roofline_hbm, "kernels": kernels, "decode_step": decode, "extra": extra,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)

@@ -75,6 +75,17 @@ def path_code(name: str) -> int:
         raise ValueError(f"unknown kernel path {name!r}; expected one of {sorted(_PATH_CODES)}") from None
 
 
+def default_state_stride(B: int, NH: int, S: int, DHQK: int, DHHV: int) -> int:
+    """The state stride the library picks for this shape when asked for 0 (read off its own workspace sizes)."""
+    lib = get_lib()
+    size = lambda s: lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 1, PATH_SPLIT, s)
+    chosen = size(0)
+    for s in range(1, 9):
+        if size(s) == chosen:
+            return s
+    raise RuntimeError("cannot determine the default state stride")
+
+
 def profile_enable(on: bool) -> None:
     get_lib().mlstm_hip_profile_enable(int(on))
 
