@@ -49,8 +49,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   constexpr int MB = MW / 32;
   constexpr int NTH = 64 * NWAVE;
   constexpr int GW = WT * NTG;     // value columns per group
-  constexpr int JL = GW > 256 ? 1 : 2;  // contraction steps (16 rows) per value slab
-  constexpr int VR = 16 * JL;      // rows per value slab
+  constexpr int VR = 8192 / GW;    // rows per value slab: a slab is 16 KB, like a score slab
   constexpr int PS = 128 + 8;      // score block row stride: P stored as Ps[n][o]
   constexpr int KS = 64 + 8;       // slab row stride of the streamed score operand
   constexpr int VS = GW + 32;      // slab row stride of the streamed value-side operand (rows 64 bytes apart in the banks)
@@ -63,6 +62,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   uint16_t* Ps = Ns + n_region;
   uint16_t* Ts = Ps + 64 * PS;
   constexpr int t_region = (128 * KS > VR * VS) ? 128 * KS : VR * VS;
+  static_assert(VR >= 16 && VR <= 128, "value slabs hold 16 to 128 rows");
   static_assert(t_region >= 32 * HS, "the slab buffer also stages 32 output rows");
   float* nvec = (float*)(Ts + t_region);  // [64] gate vector of this workgroup's positions: u_t (forward) / w_j (dV)
   float* ovec = nvec + 64;              // [128] gate vector of the source chunk: w_j (forward) / u_t (dV)
@@ -103,25 +103,94 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
     hi = (!IS_DV && sc == c) ? 2 * (nh + 1) : 4;
   };
 
-  // ---- phase 0: resident rows, gate vectors (and n_prev) into LDS; first score slab into registers
-  constexpr int KV = 128 * 8 / NTH;  // 16-byte vectors per thread per score slab (128 rows x 64 columns)
-  uint4 kreg[KV];
+  // ---- streamed operands.  The score operand (Xo rows, 64 head-dim columns per slab) and the value-side operand (Xw
+  // rows, GW columns per slab) of all source chunks form ONE sequence of steps: per source chunk DHQK/64 score slabs,
+  // then the value slabs that cover its live rows.  Every slab is 16 KB (SV 16-byte vectors per thread), so the same
+  // two register sets serve both kinds, and the slab of step s+2 is requested while step s is being multiplied: a
+  // workgroup always has two slabs on their way, whatever phase it is in.  (With one slab in flight a step cannot be
+  // shorter than a trip to the L2, several times its LDS and matrix work.)
+  constexpr int SV = 128 * 8 / NTH;      // 16-byte vectors per thread per slab
+  constexpr int VRP = NTH / (GW / 8);    // value-slab rows covered by one sweep of the workgroup
+  static_assert(SV * VRP == VR, "a value slab is as large as a score slab");
+  constexpr int OVN = NTH >= 128 ? 1 : 128 / NTH;  // gate-vector entries per thread (a workgroup may be one wave)
+  uint4 sA[SV], sB[SV];
+  float ovA[OVN], orA[OVN], ovB[OVN], orB[OVN];
   // Streamed rows are addressed as a uniform base plus a 32-bit byte offset per lane (offsets inside one (batch, head)
   // fit 32 bits, checked by the launcher), which keeps the addresses out of the vector registers.  Rows past the end
   // of the sequence are read from its last row instead of being zeroed: their gate factor is zero (forward) or the
   // value rows they meet are stored as zeros (dV), and rows of dead blocks only feed score units nobody reads.
   const char* const Xo_b = (const char*)Xo_g;
   const char* const Xw_b = (const char*)Xw_g;
-  auto load_kslab = [&](int sc, int slab) {
-    const int tv = opaque(tid);
-    const uint32_t krow0 = tv >> 3, kunit = (tv & 7) * 16;
-#pragma unroll
-    for (int v = 0; v < KV; ++v) {
-      const uint32_t t = min((uint32_t)(sc * kChunk) + krow0 + v * (NTH / 8), (uint32_t)(S - 1));
-      kreg[v] = *(const uint4*)(Xo_b + (t * (uint32_t)(DHQK * 2) + (uint32_t)(slab * 128) + kunit));
-    }
+  const int nslab = DHQK / 64;
+  // live value slabs of source chunk sc: [sl_lo, sl_hi)
+  auto vslab_range = [&](int sc, int& sl_lo, int& sl_hi) {
+    int lo, hi;
+    ob_range(sc, lo, hi);
+    sl_lo = 32 * lo / VR;
+    sl_hi = (32 * hi + VR - 1) / VR;
   };
-  load_kslab(sc_lo, 0);
+  // The two register sets alternate step by step; so that the set of a step is known at compile time, each phase
+  // (score slabs of a source chunk, value slabs of a source chunk) is padded to an even number of steps -- a padding
+  // step moves nothing and multiplies nothing.  MAYPAD is false for the shapes whose phases are even anyway.
+  constexpr bool MAYPAD_V = VR > 32;  // value phases of 64 or 128 rows per slab can be a single slab
+  const bool maypad_k = (nslab & 1) != 0;
+  const int nk2 = nslab + (nslab & 1);
+  struct Target {
+    int sc, kind, idx;  // kind 0: score slab idx; kind 1: value slab idx (absolute slab index inside the chunk)
+    bool real;
+  };
+  // the step two positions after (sc, kind, rel) in the padded sequence (rel = position inside its phase)
+  auto ahead2 = [&](int sc, int kind, int rel) {
+    int sl_lo, sl_hi;
+    vslab_range(sc, sl_lo, sl_hi);
+    const int nv = sl_hi - sl_lo, nv2 = nv + (nv & 1);
+    Target t;
+    int r2 = rel + 2;
+    if (kind == 0) {
+      if (r2 < nk2) {
+        t = {sc, 0, r2, r2 < nslab};
+      } else {
+        r2 -= nk2;
+        t = {sc, 1, sl_lo + r2, r2 < nv};
+      }
+    } else {
+      if (r2 < nv2) {
+        t = {sc, 1, sl_lo + r2, r2 < nv};
+      } else {
+        r2 -= nv2;
+        t = {sc + 1, 0, r2, sc + 1 <= sc_hi && r2 < nslab};
+      }
+    }
+    if (!t.real) t = {sc_lo, 0, 0, false};
+    return t;
+  };
+  // request a slab (and the gate vectors of its source chunk) into register set R_.  A target that is not real makes
+  // every lane request one and the same 16 bytes (a cache hit nobody waits for), so that the registers of the set are
+  // defined on every path.
+#define MLSTM_LOAD_AT(R_, OV_, OR_, grp_, tg_)                                                                       \
+  {                                                                                                                  \
+    const Target nx_ = (tg_);                                                                                        \
+    const int tl_ = opaque(tid);                                                                                     \
+    const bool isv_ = nx_.kind != 0;                                                                                 \
+    const uint32_t row0_ = isv_ ? (uint32_t)tl_ / (GW / 8) : (uint32_t)tl_ >> 3;                                     \
+    const uint32_t unit_ = nx_.real ? (isv_ ? ((uint32_t)tl_ % (GW / 8)) * 16 : ((uint32_t)tl_ & 7) * 16) : 0u;      \
+    const uint32_t rstep_ = isv_ ? VRP : NTH / 8;                                                                    \
+    const uint32_t rbase_ = (uint32_t)(nx_.sc * kChunk) + (isv_ ? (uint32_t)(VR * nx_.idx) : 0u);                    \
+    const uint32_t pitch_ = isv_ ? (uint32_t)(DHHV * 2) : (uint32_t)(DHQK * 2);                                      \
+    const uint32_t coff_ = isv_ ? (uint32_t)((grp_) * GW * 2) : (uint32_t)(nx_.idx * 128);                           \
+    const char* const base_ = isv_ ? Xw_b : Xo_b;                                                                    \
+    _Pragma("unroll") for (int v = 0; v < SV; ++v) {                                                                 \
+      const uint32_t t_ = nx_.real ? min(rbase_ + row0_ + v * rstep_, (uint32_t)(S - 1)) : rbase_;                   \
+      R_[v] = *(const uint4*)(base_ + (t_ * pitch_ + coff_ + unit_));                                                \
+    }                                                                                                                \
+    _Pragma("unroll") for (int e = 0; e < OVN; ++e) {                                                                \
+      const int idx_ = min(tl_ + e * NTH, 127);                                                                      \
+      OV_[e] = (IS_DV ? a.g.u : a.g.w)[hofs + (size_t)nx_.sc * kChunk + idx_];                                       \
+      OR_[e] = (IS_DV && a.use_nrow) ? a.nrow[hofs + (size_t)nx_.sc * kChunk + idx_] : 1.f;                          \
+    }                                                                                                                \
+  }
+  MLSTM_LOAD_AT(sA, ovA, orA, 0, (Target{sc_lo, 0, 0, true}))
+  MLSTM_LOAD_AT(sB, ovB, orB, 0, (Target{sc_lo, 0, nslab > 1 ? 1 : 0, nslab > 1}))
   // state fragments of the first contraction steps of the first column tile: requested up front, together with
   // everything else this workgroup needs first, so that all of it costs ONE trip to memory
   const int m_wave = wave * MW;  // first value column of this wave inside a column tile
@@ -189,19 +258,89 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   }
 
   constexpr int UW = 8 / NWAVE;  // score units per wave
-  constexpr int VV = VR * (GW / 8) / NTH;  // 16-byte vectors per thread per value slab (VR rows x GW columns)
-  static_assert(VV >= 1, "value slab smaller than the workgroup");
-  uint4 vreg[VV];
-  auto load_vslab = [&](int grp, int sc, int sl) {
-    const int tv = opaque(tid);
-    const uint32_t vrow0 = tv / (GW / 8), vunit = (tv % (GW / 8)) * 16;
-#pragma unroll
-    for (int v = 0; v < VV; ++v) {
-      const uint32_t t = min((uint32_t)(sc * kChunk + VR * sl) + vrow0 + v * (NTH / (GW / 8)), (uint32_t)(S - 1));
-      vreg[v] = *(const uint4*)(Xw_b + (t * (uint32_t)(DHHV * 2) + (uint32_t)(grp * GW * 2) + vunit));
-    }
-  };
-  const int nslab = DHQK / 64;
+
+  // One score-slab step with register set R_: Ts <- Xo rows x 64 head-dim columns of slab ks_; score units (32 o x 32 n;
+  // unit u = block ob_lo + u/2, position block u%2) dealt round-robin to the waves.
+#define MLSTM_K_STEP(R_, OV_, OR_, ks_)                                                                              \
+  {                                                                                                                  \
+    const bool valid_ = !maypad_k || (ks_) < nslab;                                                                  \
+    if (valid_) {                                                                                                    \
+      const int tv = opaque(tid);                                                                                    \
+      __syncthreads(); /* previous slab / output staging fully consumed */                                          \
+      _Pragma("unroll") for (int v = 0; v < SV; ++v) {                                                               \
+        const int idx = tv + v * NTH;                                                                                \
+        store_perm16(Ts + (idx >> 3) * KS, idx & 7, R_[v]);                                                          \
+      }                                                                                                              \
+      if ((ks_) == 0) {                                                                                              \
+        _Pragma("unroll") for (int e = 0; e < OVN; ++e) {                                                            \
+          const int idx = tv + e * NTH;                                                                              \
+          if (idx < 128) {                                                                                           \
+            ovec[idx] = OV_[e];                                                                                      \
+            if (IS_DV) orho[idx] = a.use_nrow ? 1.f / (OR_[e] + a.eps) : 1.f;                                        \
+          }                                                                                                          \
+        }                                                                                                            \
+      }                                                                                                              \
+      __syncthreads();                                                                                               \
+    }                                                                                                                \
+    MLSTM_LOAD_AT(R_, OV_, OR_, grp, ahead2(sc, 0, (ks_)))                                                           \
+    if (valid_) {                                                                                                    \
+      const int ln = opaque(lane);                                                                                   \
+      const int r = ln & 31, h = ln >> 5;                                                                            \
+      _Pragma("unroll") for (int k = 0; k < UW; ++k) {                                                               \
+        /* unconditional on purpose: a wave whose block lies above the diagonal multiplies rows nobody reads */    \
+        const int u = wave + k * NWAVE;                                                                              \
+        const int ob = ob_lo + (u >> 1), nb = u & 1;                                                                 \
+        const int obc = ob < 4 ? ob : 3;                                                                             \
+        _Pragma("unroll") for (int ds = 0; ds < 4; ++ds) {                                                           \
+          Frag A, B;                                                                                                 \
+          A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);                                         \
+          B.u = *(const uint4*)(Ns + (32 * nb + r) * QS + (ks_) * 64 + 16 * ds + 8 * h);                             \
+          mfma32(sacc[k], A, B);                                                                                     \
+        }                                                                                                            \
+      }                                                                                                              \
+    }                                                                                                                \
+  }
+  // One value-slab step with register set R_: Ts <- VR rows of Xw x GW columns (slab sl_lo + vs_ of the chunk);
+  // Out^T += Xw^T P over the live 16-row steps of the slab, for every value column of the group.
+#define MLSTM_V_STEP(R_, OV_, OR_, vs_)                                                                              \
+  {                                                                                                                  \
+    const bool valid_ = !MAYPAD_V || (vs_) < nv;                                                                     \
+    const int sl_ = sl_lo + (vs_);                                                                                   \
+    if (valid_) {                                                                                                    \
+      const int tv = opaque(tid);                                                                                    \
+      __syncthreads(); /* slab buffer free (first pass: P written, score slabs consumed) */                         \
+      _Pragma("unroll") for (int v = 0; v < SV; ++v) {                                                               \
+        const int j = tv / (GW / 8) + v * VRP;                                                                       \
+        const bool inside = sc * kChunk + VR * sl_ + j < S;                                                          \
+        *(uint4*)(Ts + j * VS + (tv % (GW / 8)) * 8) = inside ? R_[v] : make_uint4(0, 0, 0, 0);                      \
+      }                                                                                                              \
+      __syncthreads();                                                                                               \
+    }                                                                                                                \
+    MLSTM_LOAD_AT(R_, OV_, OR_, grp, ahead2(sc, 1, (vs_)))                                                           \
+    if (valid_) {                                                                                                    \
+      const int ln = opaque(lane);                                                                                   \
+      const int r = ln & 31, h = ln >> 5;                                                                            \
+      const int q16 = (ln >> 4) & 1, i16 = ln & 15;                                                                  \
+      const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);                                          \
+      const int row_lo = max(32 * ob_lo, VR * sl_), row_hi = min(32 * ob_hi, VR * (sl_ + 1));                        \
+      for (int row = row_lo; row < row_hi; row += 16) {                                                              \
+        const int jl = (row - VR * sl_) >> 4;                                                                        \
+        Frag B[2];                                                                                                   \
+        _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)                                                             \
+          B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + row + 8 * h);                                          \
+        _Pragma("unroll") for (int tl = 0; tl < NTG; ++tl) {                                                         \
+          Frag A[MB];                                                                                                \
+          _Pragma("unroll") for (int mb = 0; mb < MB; ++mb) {                                                        \
+            const uint16_t* p = Ts + (16 * jl + krow) * VS + (tl * WT + m_wave + 32 * mb + ncol);                    \
+            A[mb].d[0] = lds_read_tr16(p);                                                                           \
+            A[mb].d[1] = lds_read_tr16(p + 4 * VS);                                                                  \
+          }                                                                                                          \
+          _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                                                          \
+            _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32(acc[tl][mb][nb], A[mb], B[nb]);                  \
+        }                                                                                                            \
+      }                                                                                                              \
+    }                                                                                                                \
+  }
 
   for (int grp = 0; grp < NG; ++grp) {
     f32x16 acc[NTG][MB][2];
@@ -213,6 +352,11 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) acc[tl][mb][nb][i] = 0.f;
+    // later groups request their first two slabs only now (the first group's travel since the kernel started)
+    if (grp > 0) {
+      MLSTM_LOAD_AT(sA, ovA, orA, grp, (Target{sc_lo, 0, 0, true}))
+      MLSTM_LOAD_AT(sB, ovB, orB, grp, (Target{sc_lo, 0, nslab > 1 ? 1 : 0, nslab > 1}))
+    }
     __syncthreads();  // phase-0 writes visible (later groups: the previous group's output staging is stored)
     // ---- inter-chunk product, tile by tile: Out^T = State^T Xn^T
 #pragma unroll
@@ -246,127 +390,84 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
       // the next tile's first state fragments travel while this one finishes
       if (tl + 1 < NTG) MLSTM_LOAD_RING(col0 + WT)
     }
+    {
+      const int r = opaque(lane) & 31;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-      const float sc = cs[32 * nb + r];
+      for (int nb = 0; nb < 2; ++nb) {
+        const float sc = cs[32 * nb + r];
 #pragma unroll
-      for (int tl = 0; tl < NTG; ++tl)
+        for (int tl = 0; tl < NTG; ++tl)
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[tl][mb][nb] *= sc;
+          for (int mb = 0; mb < MB; ++mb) acc[tl][mb][nb] *= sc;
+      }
     }
 
     // ---- source chunks: score block, gated into Ps, then Out^T += Xw^T P for every value column of the group
     for (int sc = sc_lo; sc <= sc_hi; ++sc) {
       int ob_lo, ob_hi;
       ob_range(sc, ob_lo, ob_hi);
+      int sl_lo, sl_hi;
+      vslab_range(sc, sl_lo, sl_hi);
+      const int nv = sl_hi - sl_lo;
       const bool own = sc == c;
-      // decay between the key chunk and the query chunk of this block (0 for the own chunk)
-      float gs = 0.f;
-      for (int x = (IS_DV ? c : sc); x < (IS_DV ? sc : c); ++x) gs += graw[x];
-      // gate vectors of the source chunk: requested now, published before the first barrier of the slab loop
-      constexpr int OVN = NTH >= 128 ? 1 : 128 / NTH;  // gate-vector entries per thread (a workgroup may be one wave)
-      float ov[OVN], orh[OVN];
-#pragma unroll
-      for (int e = 0; e < OVN; ++e) {
-        const int idx = tid + e * NTH;
-        ov[e] = 0.f;
-        orh[e] = 1.f;
-        if (idx < 128) {
-          ov[e] = (IS_DV ? a.g.u : a.g.w)[hofs + (size_t)sc * kChunk + idx];
-          if (IS_DV && a.use_nrow) orh[e] = a.nrow[hofs + (size_t)sc * kChunk + idx];
-        }
-      }
-      // score units (32 o x 32 n; unit u = block ob_lo + u/2, position block u%2), dealt round-robin to the waves;
-      // contraction over DHQK in slabs of 64
       f32x16 sacc[UW];
 #pragma unroll
       for (int k = 0; k < UW; ++k)
 #pragma unroll
         for (int i = 0; i < 16; ++i) sacc[k][i] = 0.f;
-      for (int slab = 0; slab < nslab; ++slab) {
-        const int tv = opaque(tid);
-        const int r = tv & 31, h = (tv >> 5) & 1;
-        __syncthreads();  // previous slab / previous value slab / output staging fully consumed
-#pragma unroll
-        for (int v = 0; v < KV; ++v) {
-          const int idx = tv + v * NTH;
-          store_perm16(Ts + (idx >> 3) * KS, idx & 7, kreg[v]);
-        }
-        if (slab == 0) {
-#pragma unroll
-          for (int e = 0; e < OVN; ++e) {
-            const int idx = tv + e * NTH;
-            if (idx < 128) {
-              ovec[idx] = ov[e];
-              if (IS_DV) orho[idx] = a.use_nrow ? 1.f / (orh[e] + a.eps) : 1.f;
-            }
-          }
-        }
-        __syncthreads();
-        if (slab + 1 < nslab) load_kslab(sc, slab + 1);
+      for (int ks = 0; ks < nk2; ks += 2) {
+        MLSTM_K_STEP(sA, ovA, orA, ks)
+        MLSTM_K_STEP(sB, ovB, orB, ks + 1)
+      }
+      // gate, mask, round, and write P as Ps[n][o]; forward also accumulates fp32 row sums over j of the own chunk
+      {
+        // decay between the key chunk and the query chunk of this block (0 for the own chunk)
+        float gs = 0.f;
+        for (int x = (IS_DV ? c : sc); x < (IS_DV ? sc : c); ++x) gs += graw[x];
+        const int lg = opaque(lane);
+        const int r = lg & 31, h = lg >> 5;
 #pragma unroll
         for (int k = 0; k < UW; ++k) {
-          // unconditional on purpose: a wave whose block lies above the diagonal multiplies zero rows (its result is
-          // dropped at the gating step); a branch here would make the compiler shuttle the score accumulators between
-          // the two register files on every iteration
           const int u = wave + k * NWAVE;
           const int ob = ob_lo + (u >> 1), nb = u & 1;
-          const int obc = ob < 4 ? ob : 3;
+          float rsum = 0.f;
+          if (ob < ob_hi) {
+            const int nl = 32 * nb + r;    // position inside this workgroup's half
+            const int n = n0 + nl;         // position inside the chunk
+            const float un = nvec[nl] + (IS_DV ? -gs : gs);
 #pragma unroll
-          for (int ds = 0; ds < 4; ++ds) {
-            Frag A, B;
-            A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);
-            B.u = *(const uint4*)(Ns + (32 * nb + r) * QS + slab * 64 + 16 * ds + 8 * h);
-            mfma32(sacc[k], A, B);
+            for (int g4 = 0; g4 < 4; ++g4) {
+              const int o0 = 32 * ob + 8 * g4 + 4 * h;
+              const float4 xo = *(const float4*)(ovec + o0);
+              const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
+              float rho[4] = {1.f, 1.f, 1.f, 1.f};
+              if (IS_DV) {
+                const float4 rr = *(const float4*)(orho + o0);
+                rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
+              }
+              float pv[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                // exponent u_t - w_j (+ the decay between the chunks) and, in the own chunk, the causal mask j <= t
+                const float ex = IS_DV ? (xov[e] - un) : (un - xov[e]);
+                const bool keep = !own || (IS_DV ? (n <= o0 + e) : (o0 + e <= n));
+                const float val = sacc[k][4 * g4 + e] * a.qk_scale * __expf(ex) * rho[e];
+                pv[e] = keep ? val : 0.f;
+                rsum += pv[e];
+              }
+              *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+            }
+          }
+          if (!IS_DV && own && grp == 0) {
+            const float tot = rsum + __shfl_xor(rsum, 32);
+            if (h == 0) rows[u * 32 + r] = tot;  // units above the diagonal publish zero
           }
         }
       }
-      // first value slab into registers while the score block is gated
-      load_vslab(grp, sc, ob_lo * (32 / VR));
-      // gate, mask, round, and write P as Ps[n][o]; forward also accumulates fp32 row sums over j of the own chunk
-      const int lg = opaque(lane);
-#pragma unroll
-      for (int k = 0; k < UW; ++k) {
-        const int r = lg & 31, h = lg >> 5;
-        const int u = wave + k * NWAVE;
-        const int ob = ob_lo + (u >> 1), nb = u & 1;
-        float rsum = 0.f;
-        if (ob < ob_hi) {
-          const int nl = 32 * nb + r;    // position inside this workgroup's half
-          const int n = n0 + nl;         // position inside the chunk
-          const float un = nvec[nl] + (IS_DV ? -gs : gs);
-#pragma unroll
-          for (int g4 = 0; g4 < 4; ++g4) {
-            const int o0 = 32 * ob + 8 * g4 + 4 * h;
-            const float4 xo = *(const float4*)(ovec + o0);
-            const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
-            float rho[4] = {1.f, 1.f, 1.f, 1.f};
-            if (IS_DV) {
-              const float4 rr = *(const float4*)(orho + o0);
-              rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
-            }
-            float pv[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              // exponent u_t - w_j (+ the decay between the chunks) and, in the own chunk, the causal mask j <= t
-              const float ex = IS_DV ? (xov[e] - un) : (un - xov[e]);
-              const bool keep = !own || (IS_DV ? (n <= o0 + e) : (o0 + e <= n));
-              const float val = sacc[k][4 * g4 + e] * a.qk_scale * __expf(ex) * rho[e];
-              pv[e] = keep ? val : 0.f;
-              rsum += pv[e];
-            }
-            *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
-          }
-        }
-        if (!IS_DV && own && grp == 0) {
-          const float tot = rsum + __shfl_xor(rsum, 32);
-          if (h == 0) rows[u * 32 + r] = tot;  // units above the diagonal publish zero
-        }
-      }
-      __syncthreads();
 
       // ---- denominators (forward, own chunk = last source chunk, first group only); NTH/64 threads share a row
       if (!IS_DV && own && grp == 0) {
+        __syncthreads();  // row sums visible
         constexpr int TPR = NTH / 64;  // threads per row: 8, 4, 2 or 1
         const int td = opaque(tid);
         const int t = td / TPR, part = td % TPR;
@@ -406,49 +507,11 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         }
       }
 
-      // ---- Out^T += Xw^T P over the live rows of the source chunk, VR rows per slab
-      const int sl_lo = ob_lo * (32 / VR), sl_hi = ob_hi * (32 / VR);
-      for (int sl = sl_lo; sl < sl_hi; ++sl) {
-        const int tv = opaque(tid);
-        const int ln = tv & 63;
-        const int r = ln & 31, h = ln >> 5;
-        const int q16 = (ln >> 4) & 1, i16 = ln & 15;
-        const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
-        __syncthreads();  // slab buffer free (first pass: P written, score slabs consumed)
-#pragma unroll
-        for (int v = 0; v < VV; ++v) {
-          const int j = tv / (GW / 8) + v * (NTH / (GW / 8));
-          const bool inside = sc * kChunk + VR * sl + j < S;
-          *(uint4*)(Ts + j * VS + (tv % (GW / 8)) * 8) = inside ? vreg[v] : make_uint4(0, 0, 0, 0);
-        }
-        __syncthreads();
-        if (sl + 1 < sl_hi) {
-          load_vslab(grp, sc, sl + 1);
-        } else if (sc < sc_hi) {
-          load_kslab(sc + 1, 0);     // first score slab of the next source chunk
-        } else if (grp + 1 < NG) {
-          load_kslab(sc_lo, 0);      // next group starts over with the first source chunk
-        }
-#pragma unroll
-        for (int jl = 0; jl < JL; ++jl) {
-          Frag B[2];
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + VR * sl + 16 * jl + 8 * h);
-#pragma unroll
-          for (int tl = 0; tl < NTG; ++tl) {
-            Frag A[MB];
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-              const uint16_t* p = Ts + (16 * jl + krow) * VS + (tl * WT + m_wave + 32 * mb + ncol);
-              A[mb].d[0] = lds_read_tr16(p);
-              A[mb].d[1] = lds_read_tr16(p + 4 * VS);
-            }
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-              for (int nb = 0; nb < 2; ++nb) mfma32(acc[tl][mb][nb], A[mb], B[nb]);
-          }
-        }
+      // ---- Out^T += Xw^T P over the live rows of the source chunk
+      const int nv2 = nv + (nv & 1);
+      for (int vs = 0; vs < nv2; vs += 2) {
+        MLSTM_V_STEP(sA, ovA, orA, vs)
+        MLSTM_V_STEP(sB, ovB, orB, vs + 1)
       }
     }
 
@@ -488,6 +551,9 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   }
 #undef MLSTM_LOAD_RING
 #undef MLSTM_STATE_FRAG
+#undef MLSTM_LOAD_AT
+#undef MLSTM_K_STEP
+#undef MLSTM_V_STEP
 }
 
 template <int WT, int NTG, bool IS_DV, int PD, int MW>
@@ -499,7 +565,7 @@ __global__ __launch_bounds__(64 * (WT / MW))
 template <int WT, int NTG, bool IS_DV, int PD, int MW>
 static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
   constexpr int GW = WT * NTG;
-  constexpr int VR = GW > 256 ? 16 : 32;
+  constexpr int VR = 8192 / GW;
   const int QS = a.DHQK + 8;
   const size_t n_region = (size_t)64 * QS;
   const size_t t_region = (128 * 72 > VR * (GW + 32)) ? 128 * 72 : VR * (GW + 32);
