@@ -73,6 +73,21 @@ const char* mlstm_hip_last_error(void);
 #define MLSTM_PATH_FUSED 2
 
 /*
+ * head_norm: optional normalisation of every row of H over its DHHV columns, fused into the epilogue of the forward
+ * output kernel -- the op that follows the mLSTM cell in the xLSTM block and that the reference's backward convention
+ * assumes (mlstm_kernels/torch/chunkwise/native/bw.py:44-46); the reference states the norm itself in
+ * mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-35 (layer_normalize / rms_normalize: fp32
+ * reductions over the last dimension, no scale parameters).  With MLSTM_NORM_LAYER or MLSTM_NORM_RMS the forward
+ * writes the normalised rows into H (the un-normalised output never goes to memory) and the per-row mean (0 for rms)
+ * and reciprocal standard deviation into norm_mean / norm_rstd (fp32 (B,NH,S)).  Needs DHHV = 64, 128, 256 or 512 and
+ * the split kernel path.  mlstm_hip_head_norm_bw turns the gradient of the normalised rows into the gradient of H,
+ * which mlstm_hip_chunkwise_bw takes as dH.
+ */
+#define MLSTM_NORM_NONE 0
+#define MLSTM_NORM_LAYER 1
+#define MLSTM_NORM_RMS 2
+
+/*
  * Fused recurrent decode step (one token for every (b, head)).
  * Replaces: mlstm_kernels/torch/recurrent/triton_step.py:15-127 (mlstm_recurrent_step__triton_fw) and the
  * Triton kernel mlstm_kernels/triton/recurrent/fw_step_fused.py:19-195.
@@ -110,13 +125,23 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
                            void* workspace, size_t workspace_bytes, int keep_for_backward,
                            int B, int NH, int S, int DHQK, int DHHV, float eps,
                            int dtype_qkv, int dtype_gates, int gate, int normalize, int path, int state_stride,
-                           void* stream);
+                           int head_norm, float norm_eps, float* norm_mean, float* norm_rstd, void* stream);
+
+/*
+ * Backward of the fused head norm: dX = rstd * (dY - mean_D(dY) - Y * mean_D(dY * Y)) for MLSTM_NORM_LAYER,
+ * dX = rstd * (dY - Y * mean_D(dY * Y)) for MLSTM_NORM_RMS, per row of D = 64, 128, 256 or 512 values.
+ * Replaces the autograd backward of the reference's layer_normalize / rms_normalize
+ * (mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-35).  dY, Y, dX: (rows, D) in dtype (bf16);
+ * rstd: (rows) fp32 as written by the forward.
+ */
+int mlstm_hip_head_norm_bw(const void* dY, const void* Y, const float* rstd, void* dX, size_t rows, int D,
+                           int head_norm, int dtype, void* stream);
 
 /*
  * Allocation-free chunkwise forward (inference / prefill: nothing is kept for a backward pass).
  * No counterpart in the reference.  For callers that cannot allocate device memory around the call -- code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc: same arguments and results as
- * mlstm_hip_chunkwise_fw with keep_for_backward = 0, path = MLSTM_PATH_AUTO and state_stride = 0, but the workspace is
+ * mlstm_hip_chunkwise_fw with keep_for_backward = 0, path = MLSTM_PATH_AUTO, state_stride = 0 and no head norm, but the workspace is
  * a static device array of MLSTM_NOALLOC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
  * ends) instead of a caller-provided buffer.  The call allocates and frees nothing.  Shapes whose workspace
  * (mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0, MLSTM_PATH_AUTO, 0)) exceeds the static scratch are

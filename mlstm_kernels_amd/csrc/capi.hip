@@ -92,7 +92,7 @@ int set_last_error(const char* msg) { return fail(msg); }
 
 extern "C" {
 
-int mlstm_hip_abi_version(void) { return 2; }
+int mlstm_hip_abi_version(void) { return 3; }
 
 int mlstm_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
@@ -165,7 +165,8 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
                       const float* c0, const float* n0, const float* m0, void* H, float* n_out, float* m_out,
                       float* c_last, float* n_last, float* m_last, void* workspace, size_t workspace_bytes,
                       int keep_for_backward, int B, int NH, int S, int DHQK, int DHHV, float eps, int dtype_qkv,
-                      int dtype_gates, int gate, int normalize, int path, int state_stride, hipStream_t st) {
+                      int dtype_gates, int gate, int normalize, int path, int state_stride, int head_norm,
+                      float norm_eps, float* norm_mean, float* norm_rstd, hipStream_t st) {
   char msg[160];
   auto failw = [&](const char* what) {
     snprintf(msg, sizeof(msg), "%s: %s", who, what);
@@ -181,6 +182,12 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   if (has_c0 != (n0 != nullptr)) return failw("c0 and n0 must be given together");
   if (gate == MLSTM_GATE_EXP && has_c0 != (m0 != nullptr)) return failw("initial states must be given together");
   const bool fused = use_fused(path, DHQK, DHHV);
+  if (head_norm != MLSTM_NORM_NONE) {
+    if (head_norm != MLSTM_NORM_LAYER && head_norm != MLSTM_NORM_RMS) return failw("unknown head norm code");
+    if (fused) return failw("the fused kernel path has no head norm epilogue");
+    if (!mlstm::par_hv_head_norm_supported(DHHV)) return failw("the fused head norm needs DHHV = 64, 128, 256 or 512");
+    if (!norm_mean || !norm_rstd) return failw("the head norm needs its mean and rstd outputs");
+  }
   const bool with_states = keep_for_backward || !fused;
   const int stride = resolve_stride(state_stride);
   mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(workspace, B, NH, S, DHQK, DHHV, with_states, stride);
@@ -265,6 +272,10 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   pa.sig_gate = sig;
   pa.use_nrow = !(sig && !normalize);
   pa.stride = stride;
+  pa.head_norm = head_norm;
+  pa.norm_eps = norm_eps;
+  pa.norm_mean = norm_mean;
+  pa.norm_rstd = norm_rstd;
   {
     ProfileScope ps("par_h", st);
     if (const char* e = mlstm::launch_par_hv(pa, BH, /*is_dv=*/false, st)) return fail(e);
@@ -280,10 +291,26 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
                            const float* n0, const float* m0, void* H, float* n_out, float* m_out, float* c_last,
                            float* n_last, float* m_last, void* workspace, size_t workspace_bytes,
                            int keep_for_backward, int B, int NH, int S, int DHQK, int DHHV, float eps, int dtype_qkv,
-                           int dtype_gates, int gate, int normalize, int path, int state_stride, void* stream) {
+                           int dtype_gates, int gate, int normalize, int path, int state_stride, int head_norm,
+                           float norm_eps, float* norm_mean, float* norm_rstd, void* stream) {
   return chunkwise_fw_impl("mlstm_hip_chunkwise_fw", q, k, v, i, f, c0, n0, m0, H, n_out, m_out, c_last, n_last, m_last,
                            workspace, workspace_bytes, keep_for_backward, B, NH, S, DHQK, DHHV, eps, dtype_qkv,
-                           dtype_gates, gate, normalize, path, state_stride, (hipStream_t)stream);
+                           dtype_gates, gate, normalize, path, state_stride, head_norm, norm_eps, norm_mean, norm_rstd,
+                           (hipStream_t)stream);
+}
+
+int mlstm_hip_head_norm_bw(const void* dY, const void* Y, const float* rstd, void* dX, size_t rows, int D, int head_norm,
+                           int dtype, void* stream) {
+  if (!dY || !Y || !rstd || !dX) return fail("mlstm_hip_head_norm_bw: null pointer argument");
+  if (dtype != MLSTM_BF16) return fail("mlstm_hip_head_norm_bw: rows must be bf16");
+  mlstm::HeadNormBwArgs a;
+  a.dY = (const uint16_t*)dY; a.Y = (const uint16_t*)Y; a.rstd = rstd; a.dX = (uint16_t*)dX;
+  a.rows = rows; a.D = D; a.kind = head_norm;
+  {
+    ProfileScope ps("head_norm_bw", (hipStream_t)stream);
+    if (const char* e = mlstm::launch_head_norm_bw(a, (hipStream_t)stream)) return fail(e);
+  }
+  return check_launch("mlstm_hip_head_norm_bw");
 }
 
 size_t mlstm_hip_chunkwise_bw_workspace_bytes(int B, int NH, int S, int DHQK, int DHHV, int state_stride) {

@@ -42,6 +42,19 @@ struct ParHvArgs {
   int sig_gate;
   int use_nrow;             // 0 only for the un-normalised sigmoid-gate variant
   int stride;               // a chunk state is kept every `stride` chunks
+  int head_norm;            // forward: 0 none, 1 layer norm, 2 rms norm over the DHHV columns of every row of H
+  float norm_eps;
+  float* norm_mean;         // forward with head_norm: (B,NH,S) row means (0 for rms)
+  float* norm_rstd;         // forward with head_norm: (B,NH,S) reciprocal standard deviations
+};
+
+struct HeadNormBwArgs {
+  const uint16_t* dY;       // (rows, D) bf16 gradient of the normalised output
+  const uint16_t* Y;        // (rows, D) bf16 normalised output
+  const float* rstd;        // (rows)
+  uint16_t* dX;             // (rows, D) bf16 gradient of the input of the norm
+  size_t rows;
+  int D, kind;              // kind: 1 layer norm, 2 rms norm
 };
 
 struct FusedHvArgs {
@@ -96,6 +109,8 @@ const char* launch_gates(const void* i, const void* f, const float* m0, const Ga
                          int B, int NH, int S, int dtype_gates, int sig_gate, hipStream_t stream);
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream);
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream);
+bool par_hv_head_norm_supported(int DHHV);
+const char* launch_head_norm_bw(const HeadNormBwArgs& a, hipStream_t stream);
 bool fused_hv_supported(int DHQK, int DHHV);
 const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 const char* launch_par_qk_pair(const ParQkArgs& a, int BH, hipStream_t stream);

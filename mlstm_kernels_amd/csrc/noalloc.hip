@@ -72,5 +72,6 @@ extern "C" int mlstm_hip_chunkwise_fw_noalloc(const void* q, const void* k, cons
   if (ws == nullptr) return fail_noalloc(err);
   return mlstm_hip_chunkwise_fw(q, k, v, i, f, c0, n0, m0, H, n_out, m_out, c_last, n_last, m_last, ws,
                                 (size_t)MLSTM_NOALLOC_SCRATCH_BYTES, /*keep_for_backward=*/0, B, NH, S, DHQK, DHHV, eps,
-                                dtype_qkv, dtype_gates, gate, normalize, MLSTM_PATH_AUTO, /*state_stride=*/0, stream);
+                                dtype_qkv, dtype_gates, gate, normalize, MLSTM_PATH_AUTO, /*state_stride=*/0,
+                                MLSTM_NORM_NONE, 0.f, nullptr, nullptr, stream);
 }

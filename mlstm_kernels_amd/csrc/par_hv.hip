@@ -43,7 +43,7 @@ namespace mlstm {
 // PD = how many contraction steps ahead the state fragments are fetched (must divide DHQK / 16).
 // MW = value columns per wave (64 or 32): WT / MW waves share a tile.  NTG = column tiles per group (1 or 2).
 #define PAR_HV_WPE(WT_, MW_) ((WT_) / (MW_) >= 8 ? 4 : ((WT_) >= 128 ? 2 : 1))
-template <int WT, int NTG, bool IS_DV, int PD, int MW>
+template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM>
 __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId blk) {
   constexpr int NWAVE = WT / MW;   // each wave owns MW value columns of every tile of the group = MB MFMA row blocks
   constexpr int MB = MW / 32;
@@ -519,6 +519,65 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
     // would cost the registers those need).  Unconditional: after the last group the fragments of that group are
     // requested once more, cache hits nobody waits for; a conditional load would be parked in scratch memory.
     MLSTM_LOAD_RING(min(grp + 1, NG - 1) * GW)
+    // ---- optional head norm (forward only; the launcher admits it only when one group spans the whole value
+    // dimension, so that this workgroup holds complete rows of H): with x = H_t, y = (x - mean) * rsqrt(var + eps) over
+    // the DHHV columns ("layer"), or y = x * rsqrt(mean(x^2) + eps) ("rms").  Statistics in fp32 from the fp32
+    // accumulators (sum and sum of squares; x = acc * iv, so both come from the raw accumulators); each lane owns one
+    // position per 32-position block and a share of its columns, the shares of the waves meet in the slab buffer.  The
+    // result is an affine map of the accumulator, y = acc * osc + osh, applied when the rows are rounded below.
+    constexpr bool normed = !IS_DV && HEAD_NORM;
+    float osc[2] = {1.f, 1.f}, osh[2] = {0.f, 0.f};
+    if constexpr (normed) {
+      const int le = opaque(lane);
+      const int r = le & 31, h = le >> 5;
+      float* red = (float*)Ts;  // [NWAVE][2][64]
+      float p1[2], p2[2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int tl = 0; tl < NTG; ++tl)
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const float x = acc[tl][mb][nb][i];
+              s1 += x;
+              s2 += x * x;
+            }
+        p1[nb] = s1 + __shfl_xor(s1, 32);
+        p2[nb] = s2 + __shfl_xor(s2, 32);
+      }
+      __syncthreads();  // slab buffer free (last value slab consumed)
+      if (h == 0) {
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          red[wave * 128 + 32 * nb + r] = p1[nb];
+          red[wave * 128 + 64 + 32 * nb + r] = p2[nb];
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        float t1 = 0.f, t2 = 0.f;
+#pragma unroll
+        for (int w = 0; w < NWAVE; ++w) {
+          t1 += red[w * 128 + 32 * nb + r];
+          t2 += red[w * 128 + 64 + 32 * nb + r];
+        }
+        const float iv = inv[32 * nb + r];
+        const float ex = t1 * iv * (1.f / (float)DHHV), ex2 = t2 * iv * iv * (1.f / (float)DHHV);
+        const float mean = a.head_norm == 1 ? ex : 0.f;
+        const float rstd = rsqrtf(fmaxf(ex2 - mean * mean, 0.f) + a.norm_eps);
+        osc[nb] = iv * rstd;
+        osh[nb] = -mean * rstd;
+        const int tg = t_base + n0 + 32 * nb + r;
+        if (wave == 0 && h == 0 && tg < S) {
+          a.norm_mean[(size_t)bh * S + tg] = mean;
+          a.norm_rstd[(size_t)bh * S + tg] = rstd;
+        }
+      }
+    }
     // ---- epilogue: (normalise,) round, transpose through the slab buffer (32 positions at a time), coalesced store
 #pragma unroll
     for (int tl = 0; tl < NTG; ++tl) {
@@ -528,15 +587,16 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         const int le = opaque(lane);
         const int r = le & 31, h = le >> 5;
         __syncthreads();  // slab buffer free (last value slab consumed / previous half stored; inv written)
-        const float iv = IS_DV ? 1.f : inv[32 * nb + r];
+        const float iv = IS_DV ? 1.f : (normed ? osc[nb] : inv[32 * nb + r]);
+        const float sh = normed ? osh[nb] : 0.f;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
           for (int g4 = 0; g4 < 4; ++g4) {
             const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
             *(uint2*)(Ts + r * HS + w0) =
-                make_uint2(pack_bf16x2(acc[tl][mb][nb][4 * g4 + 0] * iv, acc[tl][mb][nb][4 * g4 + 1] * iv),
-                           pack_bf16x2(acc[tl][mb][nb][4 * g4 + 2] * iv, acc[tl][mb][nb][4 * g4 + 3] * iv));
+                make_uint2(pack_bf16x2(acc[tl][mb][nb][4 * g4 + 0] * iv + sh, acc[tl][mb][nb][4 * g4 + 1] * iv + sh),
+                           pack_bf16x2(acc[tl][mb][nb][4 * g4 + 2] * iv + sh, acc[tl][mb][nb][4 * g4 + 3] * iv + sh));
           }
         __syncthreads();
         constexpr int vec_per_row = WT / 8;
@@ -556,14 +616,14 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
 #undef MLSTM_V_STEP
 }
 
-template <int WT, int NTG, bool IS_DV, int PD, int MW>
+template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM>
 __global__ __launch_bounds__(64 * (WT / MW))
     __attribute__((amdgpu_waves_per_eu(PAR_HV_WPE(WT, MW), PAR_HV_WPE(WT, MW)))) void par_hv_kernel(ParHvArgs a) {
-  par_hv_body<WT, NTG, IS_DV, PD, MW>(a, xcd_block_id());  // the workgroups that share a kept state run on one XCD
+  par_hv_body<WT, NTG, IS_DV, PD, MW, HEAD_NORM>(a, xcd_block_id());  // the workgroups that share a kept state run on one XCD
 }
 
-template <int WT, int NTG, bool IS_DV, int PD, int MW>
-static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
+template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM>
+static const char* launch_par_hv_hn(const ParHvArgs& a, int BH, hipStream_t stream) {
   constexpr int GW = WT * NTG;
   constexpr int VR = 8192 / GW;
   const int QS = a.DHQK + 8;
@@ -573,12 +633,20 @@ static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stre
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
   if ((size_t)a.S * (size_t)(a.DHHV > a.DHQK ? a.DHHV : a.DHQK) * 2 >= ((size_t)1 << 32))
     return "par_hv: one (batch, head) slab of an input exceeds 4 GiB";
-  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, NTG, IS_DV, PD, MW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, NTG, IS_DV, PD, MW, HEAD_NORM>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_hv: cannot raise the dynamic LDS limit";
   dim3 grid(2, a.NC, BH);
-  hipLaunchKernelGGL((par_hv_kernel<WT, NTG, IS_DV, PD, MW>), grid, dim3(64 * (WT / MW)), smem, stream, a);
+  hipLaunchKernelGGL((par_hv_kernel<WT, NTG, IS_DV, PD, MW, HEAD_NORM>), grid, dim3(64 * (WT / MW)), smem, stream, a);
   return nullptr;
+}
+
+template <int WT, int NTG, bool IS_DV, int PD, int MW>
+static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
+  if constexpr (!IS_DV) {
+    if (a.head_norm != 0) return launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, true>(a, BH, stream);
+  }
+  return launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, false>(a, BH, stream);
 }
 
 template <int WT, int NTG, bool IS_DV>
@@ -597,9 +665,18 @@ static const char* launch_par_hv_d(const ParHvArgs& a, int BH, hipStream_t strea
   return launch_par_hv_t<64, 1, IS_DV>(a, BH, stream);
 }
 
+// one workgroup holds complete rows of H only when a single group of column tiles spans the value dimension
+bool par_hv_head_norm_supported(int DHHV) { return DHHV == 64 || DHHV == 128 || DHHV == 256 || DHHV == 512; }
+
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
   if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "par_hv: DHQK and DHHV must be multiples of 64";
   if (a.stride < 1 || a.stride > kMaxStateStride) return "par_hv: state stride out of range";
+  if (a.head_norm != 0) {
+    if (is_dv) return "par_hv: the head norm belongs to the forward output";
+    if (a.head_norm != 1 && a.head_norm != 2) return "par_hv: unknown head norm code";
+    if (!par_hv_head_norm_supported(a.DHHV)) return "par_hv: the fused head norm needs DHHV = 64, 128, 256 or 512";
+    if (a.norm_mean == nullptr || a.norm_rstd == nullptr) return "par_hv: the head norm needs its mean / rstd outputs";
+  }
   return is_dv ? launch_par_hv_d<true>(a, BH, stream) : launch_par_hv_d<false>(a, BH, stream);
 }
 

@@ -76,7 +76,7 @@ def validate_xl_chunk_shapes(S: int, chunk_size: int) -> None:
     assert S % chunk_size == 0, f"Sequence length must be divisible by the target chunk size {chunk_size}."
 
 
-def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep, path, stride):
+def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep, path, stride, norm=0, norm_eps=1e-6):
     B, NH, S, DHQK = q.shape
     DHHV = v.shape[-1]
     dev = q.device
@@ -93,6 +93,13 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
         )
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
+    if norm != _lib.NORM_NONE:
+        if DHHV not in (64, 128, 256, 512):
+            raise ValueError(f"the fused head norm needs DHHV = 64, 128, 256 or 512, got {DHHV}")
+        norm_mean = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
+        norm_rstd = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
+    else:
+        norm_mean = norm_rstd = None
     if want_last:
         c_last = torch.empty(B, NH, DHQK, DHHV, dtype=torch.float32, device=dev)
         n_last = torch.empty(B, NH, DHQK, dtype=torch.float32, device=dev)
@@ -104,10 +111,10 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
         ptr(H), None, None, ptr(c_last), ptr(n_last), ptr(m_last),
         ptr(ws), ws_bytes, int(keep), B, NH, S, DHQK, DHHV, float(eps),
         _lib.BF16, dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
-        current_stream_ptr(dev),
+        norm, float(norm_eps), ptr(norm_mean), ptr(norm_rstd), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_chunkwise_fw")
-    return H, c_last, n_last, m_last, ws
+    return H, c_last, n_last, m_last, ws, norm_rstd
 
 
 def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
@@ -135,7 +142,7 @@ def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
     return dev, qb, kb, vb, ib, fb, c0, n0, m0
 
 
-def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, stride: int):
+def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, stride: int, norm: int, norm_eps: float):
     class _HipChunkwiseFwBw(torch.autograd.Function):
         @staticmethod
         @custom_fwd(device_type="cuda", cast_inputs=autocast_kernel_dtype)
@@ -146,10 +153,14 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
             out_dtype = q.dtype
             dev, qb, kb, vb, ib, fb, c0f, n0f, m0f = _prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
             needs_bw = any(ctx.needs_input_grad[:6])
-            H, c_last, n_last, m_last, ws = _fw_launch(
-                qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw, path, stride
+            H, c_last, n_last, m_last, ws, norm_rstd = _fw_launch(
+                qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw, path, stride,
+                norm, norm_eps
             )
-            ctx.save_for_backward(qb, kb, vb, ib, fb, ws)
+            if norm != _lib.NORM_NONE and needs_bw:
+                ctx.save_for_backward(qb, kb, vb, ib, fb, ws, H, norm_rstd)   # H holds the normalised rows
+            else:
+                ctx.save_for_backward(qb, kb, vb, ib, fb, ws)
             ctx.cfg = (eps, q.dtype, k.dtype, v.dtype, i.dtype, f.dtype,
                        None if c0 is None else c0.dtype, n0 is not None, m0 is not None)
             H = H if out_dtype == torch.bfloat16 else H.to(out_dtype)
@@ -158,7 +169,7 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
         @staticmethod
         @custom_bwd(device_type="cuda")
         def backward(ctx, dH, dC_last, dn_last, dm_last):
-            qb, kb, vb, ib, fb, ws = ctx.saved_tensors
+            qb, kb, vb, ib, fb, ws, *normed = ctx.saved_tensors
             eps, qdt, kdt, vdt, idt, fdt, c0dt, has_n0, has_m0 = ctx.cfg
             B, NH, S, DHQK = qb.shape
             DHHV = vb.shape[-1]
@@ -169,6 +180,14 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
             if dH is None:  # only the last states are differentiated
                 dH = torch.zeros(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
             dHb = dH.to(torch.bfloat16).contiguous()
+            if normed:
+                # gradient of the normalised rows -> gradient of H (the un-normalised rows were never stored)
+                Hn, rstd = normed
+                dHraw = torch.empty_like(dHb)
+                rc = lib.mlstm_hip_head_norm_bw(ptr(dHb), ptr(Hn), ptr(rstd), ptr(dHraw), B * NH * S, DHHV, norm,
+                                                _lib.BF16, current_stream_ptr(dev))
+                _lib.check(rc, "mlstm_hip_head_norm_bw")
+                dHb = dHraw
             dCl = None if dC_last is None else dC_last.to(torch.float32).contiguous()
             dQ, dK, dV = torch.empty_like(qb), torch.empty_like(kb), torch.empty_like(vb)
             dI = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
@@ -193,13 +212,17 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
 _FWBW_CACHE: dict = {}
 
 
-def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool, kernel_path: str, stride: int):
+def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool, kernel_path: str, stride: int,
+              head_norm: str = "none", head_norm_eps: float = 1e-6):
     if autocast_kernel_dtype not in (torch.float32, torch.float16, torch.bfloat16):
         raise ValueError(f"Unsupported kernel dtype {autocast_kernel_dtype}.")
     path = _lib.path_code(kernel_path)
-    key = (autocast_kernel_dtype, siging, normalize, path, stride)
+    norm = _lib.norm_code(head_norm)
+    if norm != _lib.NORM_NONE and path == _lib.PATH_FUSED:
+        raise ValueError("head_norm is fused into the split kernel path only (kernel_path='auto' or 'split')")
+    key = (autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps))
     if key not in _FWBW_CACHE:
-        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize, path, stride)
+        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps))
     return _FWBW_CACHE[key]
 
 
@@ -218,6 +241,8 @@ def mlstm_chunkwise__hip_xl_chunk(
     autocast_kernel_dtype: torch.dtype = torch.float32,
     any_sequence_length: bool = False,
     kernel_path: str = "auto",
+    head_norm: str = "none",
+    head_norm_eps: float = 1e-6,
     **tuning_kwargs,
 ):
     """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
@@ -227,11 +252,15 @@ def mlstm_chunkwise__hip_xl_chunk(
     ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
     tail themselves, so every S >= 1 is one call.  ``kernel_path`` ("auto", "split", "fused"; not in the reference)
     selects the kernels of the value-column side.  ``chunk_size_intra`` (reference keyword) sets the distance between
-    kept chunk states."""
+    kept chunk states.  ``head_norm`` ("none", "layer", "rms"; not in the reference's operator) fuses the multi-head
+    norm that follows the cell in the xLSTM block -- the reference's ``apply_normalize(norm_specifier, x, eps)``,
+    mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-64, over the DHHV columns of every row, without
+    scale parameters -- into the output kernel: the returned ``H`` is then the normalised one and the un-normalised
+    output never goes to memory (DHHV = 64, 128, 256 or 512)."""
     stride = _state_stride(tuning_kwargs, "mlstm_chunkwise__hip_xl_chunk")
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
-    fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride)
+    fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride, head_norm, head_norm_eps)
     H, c_last, n_last, m_last = fn.apply(q, k, v, i, f, c_initial, n_initial, m_initial, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last, m_last)
@@ -254,14 +283,16 @@ def mlstm_siging_chunkwise__hip_xl_chunk(
     autocast_kernel_dtype: torch.dtype = torch.float32,
     any_sequence_length: bool = False,
     kernel_path: str = "auto",
+    head_norm: str = "none",
+    head_norm_eps: float = 1e-6,
     **tuning_kwargs,
 ):
     """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``.
-    ``any_sequence_length``, ``kernel_path`` and ``chunk_size_intra`` as for the exp gate."""
+    ``any_sequence_length``, ``kernel_path``, ``chunk_size_intra`` and ``head_norm`` as for the exp gate."""
     stride = _state_stride(tuning_kwargs, "mlstm_siging_chunkwise__hip_xl_chunk")
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
-    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride)
+    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride, head_norm, head_norm_eps)
     H, c_last, n_last, _ = fn.apply(q, k, v, i, f, c_initial, n_initial, None, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last)

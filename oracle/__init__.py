@@ -17,7 +17,14 @@ What pins each function (none of them is pinned by retyping its own formula):
 * sigmoid-input-gate variants                  -- recurrent sig loop == quadratic sig == chunkwise sig,
   detached-normaliser autograd for the gradients, state passing for non-zero initial (C, n).
 
-The reference ships no golden vectors for this path (its tests compare live implementations), so the
-fixtures under tests/golden/ are closed-form known answers plus a regression dump of this oracle.
+* ``head_normalize`` / ``head_normalize_bw``    -- torch.nn.functional.layer_norm / rms formula and fp64 autograd
+  (tests/test_oracle.py).
+* ``H_abs`` / ``d*_abs`` magnitude sums (``return_bounds``) are derived quantities for the test bounds, not part of
+  the reference's algorithm.
+
+The reference ships no golden vectors for this path (its tests compare live implementations).  The fixtures under
+tests/golden/ are: closed-form known answers, a regression dump of this oracle, and vectors written from the
+reference's OWN native functions (chunkwise forward/backward, quadratic sigmoid-gate forward/backward, decode step)
+by the two make_reference_vectors*.py scripts; the oracle reproduces all of them to 1e-5.
 """
 from .mlstm_ref import *  # noqa: F401,F403

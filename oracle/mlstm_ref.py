@@ -42,6 +42,8 @@ __all__ = [
     "parallel_siging_bw",
     "chunkwise_fw",
     "chunkwise_bw",
+    "head_normalize",
+    "head_normalize_bw",
     "mlstm_chunkwise__native_autograd",
     "mlstm_chunkwise__native_custbw",
     "mlstm_siging_chunkwise__native_custbw",
@@ -349,6 +351,38 @@ def chunkwise_bw(q, k, v, i, f, dH, c_initial=None, n_initial=None, m_initial=No
     if return_bounds:
         return dQ, dK, dV, dI, dF, (dC if c_initial is not None else None), {"dQ_abs": dQa, "dK_abs": dKa, "dV_abs": dVa}
     return dQ, dK, dV, dI, dF, (dC if c_initial is not None else None)
+
+
+# --------------------------------------------------------------------------------------------------
+# head norm (the op that follows the cell in the xLSTM block)
+# --------------------------------------------------------------------------------------------------
+def head_normalize(x, norm_specifier: str = "layer", eps: float = 1e-6):
+    """Normalisation over the last dimension without scale parameters, as the reference states it in
+    mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-64 (``apply_normalize``):
+    "layer": (x - mean) * rsqrt(biased var + eps)  (:23-34);  "rms": x * rsqrt(mean(x^2) + eps)  (:11-20);
+    "none": x.  Computed in the dtype of x (the tests feed fp64)."""
+    if norm_specifier == "none":
+        return x
+    if norm_specifier == "rms":
+        return x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+    if norm_specifier == "layer":
+        xc = x - x.mean(dim=-1, keepdim=True)
+        return xc * torch.rsqrt(x.var(dim=-1, keepdim=True, unbiased=False) + eps)
+    raise ValueError(f"Unsupported norm specifier {norm_specifier}.")
+
+
+def head_normalize_bw(dy, x, norm_specifier: str = "layer", eps: float = 1e-6):
+    """Gradient of ``head_normalize`` with respect to x, in closed form (checked against autograd in the tests):
+    with y = head_normalize(x) and rstd the reciprocal root above,
+    "layer": rstd * (dy - mean(dy) - y * mean(dy * y));  "rms": rstd * (dy - y * mean(dy * y))."""
+    if norm_specifier == "none":
+        return dy
+    y = head_normalize(x, norm_specifier, eps)
+    if norm_specifier == "rms":
+        rstd = torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps)
+        return rstd * (dy - y * (dy * y).mean(dim=-1, keepdim=True))
+    rstd = torch.rsqrt(x.var(dim=-1, keepdim=True, unbiased=False) + eps)
+    return rstd * (dy - dy.mean(dim=-1, keepdim=True) - y * (dy * y).mean(dim=-1, keepdim=True))
 
 
 # --------------------------------------------------------------------------------------------------

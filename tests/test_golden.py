@@ -129,7 +129,8 @@ def test_hip_stored_rows_match_reference_native_vectors(case):
     m_out = torch.empty(B, NH, S, dtype=torch.float32, device=dev)
     rc = lib.mlstm_hip_chunkwise_fw(ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0), ptr(H), ptr(n_out),
                                     ptr(m_out), None, None, None, ptr(ws), ws_bytes, 0, B, NH, S, DHQK, DHHV, 1e-6,
-                                    _lib.BF16, _lib.F32, _lib.GATE_EXP, 1, _lib.PATH_AUTO, 0, current_stream_ptr(dev))
+                                    _lib.BF16, _lib.F32, _lib.GATE_EXP, 1, _lib.PATH_AUTO, 0, _lib.NORM_NONE, 0.0, None, None,
+                                    current_stream_ptr(dev))
     _lib.check(rc, "mlstm_hip_chunkwise_fw")
     torch.cuda.synchronize()
     assert (m_out.cpu() - z["m_out"]).abs().max() <= 1e-4

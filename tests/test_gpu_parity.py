@@ -480,3 +480,45 @@ def test_backend_module_hip_train_and_inference():
     Hs, (Cs, ns) = sig(qq, kk, vv, ii, ff)
     Hs_r, _ = O.parallel_siging_fw(*(d64(t[:, :, :256]) for t in (q, k, v, i, f)), normalize=False)
     check_matrix(Hs, Hs_r, "H (sig, not normalised)")
+
+
+# ------------------------------------------------------------------------------------------ fused head norm
+@pytest.mark.parametrize("spec", ["layer", "rms"])
+@pytest.mark.parametrize("B,NH,S,DQK,DHV,siging", [(1, 2, 384, 256, 512, False), (2, 2, 200, 64, 128, False),
+                                                   (1, 2, 256, 128, 256, True), (1, 1, 128, 64, 64, False)])
+def test_fused_head_norm_forward_backward(spec, B, NH, S, DQK, DHV, siging, kernel_variant):
+    """The head norm fused into the output kernel (and its backward kernel) against the oracle's cell followed by the
+    oracle's norm: Hn = norm(H); gradients of sum(Hn * dY) through norm and cell.  Normalised rows are O(1), so the
+    comparison is 2e-2 absolute/relative on >= 99.9 % of the elements and 1e-2 norm-wise; the un-normalised H is
+    never written, the saved statistics are checked directly."""
+    if kernel_variant.startswith("fused"):
+        pytest.skip("the head norm is fused into the split path's output kernel")
+    exp_op, sig_op, *_ = _ops()
+    op = sig_op if siging else exp_op
+    q, k, v, i, f = make_qkvif(B, NH, S, DQK, DHV, seed=S + DHV)
+    g = torch.Generator().manual_seed(3)
+    dY = torch.randn(B, NH, S, DHV, generator=g).bfloat16()
+    L = next(c for c in (128, 64, 32, 16, 8) if S % c == 0)
+    fw = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=L, siging=siging)
+    Hn_ref = O.head_normalize(fw["H"], spec, eps=1e-6)
+    dH_ref = O.head_normalize_bw(d64(dY), fw["H"], spec, eps=1e-6)
+    bw = O.chunkwise_bw(*(d64(t) for t in (q, k, v, i, f)), dH_ref, chunk_size=L, siging=siging)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (q, k, v, i, f)]
+    Hn, st = op(*leaves, return_last_states=True, chunk_size=128, any_sequence_length=True, head_norm=spec, head_norm_eps=1e-6)
+    (Hn.float() * dY.to(DEV).float()).sum().backward()
+    assert Hn.dtype == torch.bfloat16 and Hn.shape == v.shape
+    check_matrix(Hn, Hn_ref, "Hn", frac=1e-3, scale_tol=2e-2, norm_tol=1e-2)
+    assert_state_close(st[0], fw["C_last"], 1e-3, "C_last")
+    for name, leaf, r_ in zip(["dQ", "dK", "dV"], leaves[:3], bw[:3]):
+        check_matrix(leaf.grad, r_, name, frac=2e-3, scale_tol=2e-2, norm_tol=1e-2)
+    for name, leaf, r_ in zip(["dI", "dF"], leaves[3:], bw[3:5]):
+        assert rel_to_scale(leaf.grad, r_) <= 5e-2, name
+
+
+def test_fused_head_norm_rejects_unsupported_value_dimension():
+    exp_op, *_ = _ops()
+    q, k, v, i, f = make_qkvif(1, 1, 128, 64, 192)
+    with pytest.raises(ValueError, match="fused head norm needs DHHV"):
+        exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128, head_norm="layer", kernel_path="split")
+    with pytest.raises(ValueError, match="Unsupported norm specifier"):
+        exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128, head_norm="batch", kernel_path="split")

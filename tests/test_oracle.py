@@ -251,3 +251,26 @@ def test_custbw_wrapper_autograd_plumbing():
     ref = O.chunkwise_bw(q, k, v, i, f, dH, chunk_size=16)
     for leaf, r in zip(leaves, ref[:5]):
         torch.testing.assert_close(leaf.grad, r)
+
+
+# ------------------------------------------------------------------ head norm
+@pytest.mark.parametrize("spec", ["layer", "rms"])
+def test_head_normalize_matches_library_routine_and_autograd(spec):
+    """The oracle's head norm against torch's own layer_norm (rms: the textbook formula on a hand-made row), and its
+    closed-form gradient against fp64 autograd."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 3, 5, 64, generator=g, dtype=torch.float64) * 2 + 0.3
+    y = O.head_normalize(x, spec, eps=1e-6)
+    if spec == "layer":
+        torch.testing.assert_close(y, torch.nn.functional.layer_norm(x, (64,), eps=1e-6), rtol=1e-12, atol=1e-12)
+    else:
+        row = torch.tensor([[3.0, -4.0]], dtype=torch.float64)           # rms = sqrt(12.5)
+        torch.testing.assert_close(O.head_normalize(row, "rms", eps=0.0), row / 12.5 ** 0.5, rtol=1e-14, atol=1e-14)
+        torch.testing.assert_close((y * y).mean(-1), torch.ones(2, 3, 5, dtype=torch.float64), rtol=1e-5, atol=1e-5)
+    xr = x.clone().requires_grad_(True)
+    dy = torch.randn(2, 3, 5, 64, generator=g, dtype=torch.float64)
+    (O.head_normalize(xr, spec, eps=1e-6) * dy).sum().backward()
+    torch.testing.assert_close(O.head_normalize_bw(dy, x, spec, eps=1e-6), xr.grad, rtol=1e-10, atol=1e-10)
+    assert O.head_normalize(x, "none") is x
+    with pytest.raises(ValueError):
+        O.head_normalize(x, "batch")

@@ -37,7 +37,8 @@ def _call_both(B, NH, S, DHQK, DHHV, seed, gate, init):
             ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0, _lib.PATH_AUTO, 0)
             assert 0 < ws_bytes <= _lib.NOALLOC_SCRATCH_BYTES
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-            rc = lib.mlstm_hip_chunkwise_fw(*head, ptr(ws), ws_bytes, 0, *tail, _lib.PATH_AUTO, 0, current_stream_ptr(dev))
+            rc = lib.mlstm_hip_chunkwise_fw(*head, ptr(ws), ws_bytes, 0, *tail, _lib.PATH_AUTO, 0, _lib.NORM_NONE, 0.0, None, None,
+                                    current_stream_ptr(dev))
             _lib.check(rc, "mlstm_hip_chunkwise_fw")
         torch.cuda.synchronize()
         outs.append((H, n_out, m_out, c_last, n_last, m_last))
