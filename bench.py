@@ -20,7 +20,8 @@ Objects on the JSON line besides the contract's keys:
   roofline_hbm  -- the same kernel against the HBM peak (algorithmic bytes per launch).
   kernels       -- average duration, algorithmic TFLOP/s and GB/s of every kernel of the step.
   decode_step   -- fused decode step at B=256 after a chunkwise prefill of 2048 positions: ms per step, algorithmic
-                   GB/s, its own HBM roofline; B=64 and B=16 (whose state fits the memory-side cache: "bound": "mall").
+                   GB/s, its own HBM roofline; B=64 and B=16 (whose state fits the memory-side cache: "bound": "mall");
+                   multi_token: 128 tokens per (batch, head) in ONE launch of the multi-token kernel.
   extra         -- the other BASELINE configurations, same protocol: B=16/S=4096 and B=64/S=1024 (fwd+bwd), the
                    sigmoid gate with a non-zero initial state at B=4/S=16384, forward-only at B=4/S=16384, and the
                    latter two shapes with the multi-head layer norm fused into the output kernel.
@@ -349,9 +350,32 @@ def main():
                          "traffic": traffic.get("step") if Bd == DECODE_B else None},
         }
 
+    # ---- multi-token decode: DECODE_STEPS tokens in one launch, the state stays on chip between tokens
+    def bench_decode_sequence(Bd):
+        from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_sequence__hip
+        T = DECODE_STEPS
+        qs, ks, vs = rn(Bd, NH, T, DHQK).bfloat16(), rn(Bd, NH, T, DHQK).bfloat16(), rn(Bd, NH, T, DHHV).bfloat16()
+        is_, fs = rn(Bd, NH, T), 3 + rn(Bd, NH, T)
+        c, n, m = rn(Bd, NH, DHQK, DHHV), rn(Bd, NH, DHQK), rn(Bd, NH, 1)
+        times = []
+        for rep in range(4):
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            mlstm_recurrent_sequence__hip(qs, ks, vs, is_, fs, c, n, m, return_last_states=True)
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1))
+        ms = sorted(times[1:])[1]
+        return {"batch": Bd, "tokens": T, "mode": "one launch for all tokens (state read and written once)",
+                "ms_total": round(ms, 4), "us_per_token": round(ms / T * 1e3, 3),
+                "tokens_per_s": round(Bd * T / (ms * 1e-3), 1),
+                "state_bytes_moved": 2 * Bd * NH * DHQK * DHHV * 4}
+
     decode = bench_decode(DECODE_B, graph=False)
     if not args.no_extra:
         decode["other_batches"] = [bench_decode(b, graph=g_) for b in (64, 16) for g_ in (False, True)]
+        decode["multi_token"] = [bench_decode_sequence(b) for b in (DECODE_B, 64, 16)]
     torch.cuda.empty_cache()
 
     out = {

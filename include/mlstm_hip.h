@@ -102,6 +102,22 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
                    int dtype_qkv, int dtype_gates, void* stream);
 
 /*
+ * Recurrent mLSTM over T tokens in one launch (multi-token decode, the remainder of a prefill): the step above
+ * applied T times with the state held on chip -- C is read once before the first token and written once after the
+ * last, instead of once each way per token.
+ * Replaces: the token loop mlstm_kernels/torch/recurrent/native_sequence.py:13-122
+ * (mlstm_recurrent_sequence__triton_step_fused_fw = _mlstm_recurrent_sequence_loop_fw over the fused step).
+ *   q,k (B,NH,T,DHQK), v (B,NH,T,DHHV) in dtype_qkv; i,f (B,NH,T) in dtype_gates; h (B,NH,T,DHHV) in dtype_qkv;
+ *   states as for mlstm_hip_step (c_out may alias c_in, n_out/m_out must be distinct from n_in/m_in).
+ *   DHQK <= 1024.
+ */
+int mlstm_hip_recurrent_sequence(const void* q, const void* k, const void* v, const void* i, const void* f,
+                                 const float* c_in, const float* n_in, const float* m_in,
+                                 void* h, float* c_out, float* n_out, float* m_out,
+                                 int B, int NH, int T, int DHQK, int DHHV, float eps,
+                                 int dtype_qkv, int dtype_gates, void* stream);
+
+/*
  * Bytes of caller-provided workspace the chunkwise forward needs.  With keep_for_backward != 0 the
  * workspace additionally holds everything the backward re-uses (gate vectors, per-chunk bf16 states,
  * per-row normalisers) and must be handed unchanged to mlstm_hip_chunkwise_bw.

@@ -104,30 +104,43 @@ def mlstm_recurrent_sequence__hip(
     dtype_state: torch.dtype = torch.float32,
     **kwargs,
 ):
-    """Token loop over the HIP step (used for the short remainder of a prefill).  The state is updated in
-    place in one C buffer; n and m ping-pong between two small buffers."""
+    """All S tokens in one launch of the multi-token kernel: the state stays on chip between tokens and moves
+    through HBM once each way for the whole sequence (a loop of single steps moves it once each way per token).
+    Used for multi-token decode and for the short remainder of a prefill.  Same arguments and return structure
+    as mlstm_recurrent_sequence__triton_step_fused_fw (mlstm_kernels/torch/recurrent/native_sequence.py:86-122)."""
     B, NH, S, DHQK = q.shape
     DHHV = v.shape[-1]
+    assert k.shape == q.shape, "q and k must have the same shape"
+    assert v.shape[:3] == (B, NH, S), f"v has wrong shape, got {v.shape}"
+    assert i.shape == (B, NH, S) and f.shape == (B, NH, S), "i and f must have shape (B, NH, S)"
+    if dtype_state != torch.float32:
+        raise NotImplementedError("the HIP step kernels keep the recurrent state in float32")
     dev = require_gpu(q, k, v, i, f)
     if c_initial is not None:
         assert n_initial is not None and m_initial is not None, "Initial states must be provided together."
-        c = c_initial.to(torch.float32).clone()
-        n = n_initial.to(torch.float32).clone()
-        m = m_initial.to(torch.float32).clone().reshape(B, NH, 1)
+        c = c_initial.to(torch.float32).contiguous()
+        n = n_initial.to(torch.float32).contiguous()
+        m = m_initial.to(torch.float32).contiguous().reshape(B, NH, 1)
+        assert c.shape == (B, NH, DHQK, DHHV), f"c_initial has wrong shape, got {c.shape}"
+        assert n.shape == (B, NH, DHQK), f"n_initial has wrong shape, got {n.shape}"
     else:
         c = torch.zeros(B, NH, DHQK, DHHV, dtype=torch.float32, device=dev)
         n = torch.zeros(B, NH, DHQK, dtype=torch.float32, device=dev)
         m = torch.zeros(B, NH, 1, dtype=torch.float32, device=dev)
-    n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
-    hs = []
-    for t in range(S):
-        h, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(
-            c, n, m, q[:, :, t], k[:, :, t], v[:, :, t], i[:, :, t, None], f[:, :, t, None],
-            matC_new=c, vecN_new=n_alt, scaM_new=m_alt, eps=eps, dtype_state=dtype_state,
-        )
-        n_alt, m_alt, n, m = n, m, n_new, m_new
-        hs.append(h)
-    H = torch.stack(hs, dim=-2)
+    if S == 0:
+        H = torch.empty(B, NH, 0, DHHV, dtype=q.dtype, device=dev)
+        return (H, (c.clone(), n.clone(), m.clone())) if return_last_states else H
+    qc, kc, vc = q.contiguous(), k.to(q.dtype).contiguous(), v.to(q.dtype).contiguous()
+    ic, fc = i.contiguous(), f.to(i.dtype).contiguous()
+    H = torch.empty(B, NH, S, DHHV, dtype=q.dtype, device=dev)
+    c_out, n_out, m_out = torch.empty_like(c), torch.empty_like(n), torch.empty_like(m)
+    lib = _lib.get_lib()
+    rc = lib.mlstm_hip_recurrent_sequence(
+        ptr(qc), ptr(kc), ptr(vc), ptr(ic), ptr(fc), ptr(c), ptr(n), ptr(m),
+        ptr(H), ptr(c_out), ptr(n_out), ptr(m_out),
+        B, NH, S, DHQK, DHHV, float(eps), dtype_code(qc), dtype_code(ic), current_stream_ptr(dev),
+    )
+    _lib.check(rc, "mlstm_hip_recurrent_sequence")
     if return_last_states:
-        return H, (c, n, m)
+        return H, (c_out, n_out, m_out)
     return H

@@ -149,6 +149,62 @@ def test_step_parity(B, NH, DQK, DHV, dtype):
     assert c3.data_ptr() == c_dev.data_ptr() and torch.equal(c3, c2) and torch.equal(h3, h)
 
 
+@pytest.mark.parametrize("B,NH,T,DQK,DHV", [
+    (2, 2, 1, 64, 128), (3, 4, 7, 256, 512), (1, 1, 33, 128, 192), (2, 3, 64, 384, 512),
+    (3, 2, 5, 96, 100), (1, 1, 9, 48, 36), (2, 2, 6, 130, 260), (2, 1, 300, 64, 64), (1, 2, 4, 640, 64), (16, 8, 16, 256, 512),
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("init", [False, True])
+def test_recurrent_sequence_parity(B, NH, T, DQK, DHV, dtype, init):
+    """T tokens in one launch of the multi-token kernel against the oracle's fp64 token loop, and against a loop of
+    single-step launches of the product (same arithmetic per element of the state: C, n, m must agree to rounding)."""
+    *_, step, seq = _ops()
+    g = torch.Generator().manual_seed(11 + T)
+    q, k, v = (torch.randn(B, NH, T, d, generator=g).to(dtype) for d in (DQK, DQK, DHV))
+    i, f = torch.randn(B, NH, T, generator=g), 3 + torch.randn(B, NH, T, generator=g)
+    st = None
+    if init:
+        st = (torch.randn(B, NH, DQK, DHV, generator=g), torch.randn(B, NH, DQK, generator=g), torch.randn(B, NH, 1, generator=g))
+    kw_r = {} if st is None else dict(c_initial=d64(st[0]), n_initial=d64(st[1]), m_initial=d64(st[2]))
+    H_r, (c_r, n_r, m_r) = O.recurrent_sequence(*(d64(t) for t in (q, k, v, i, f)), **kw_r)
+    kw = {} if st is None else dict(c_initial=st[0].to(DEV), n_initial=st[1].to(DEV), m_initial=st[2].to(DEV))
+    c0_before = None if st is None else kw["c_initial"].clone()
+    H, (c2, n2, m2) = seq(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, **kw)
+    assert H.shape == (B, NH, T, DHV) and H.dtype == dtype and c2.dtype == torch.float32
+    assert rel_to_scale(H, H_r) <= (5e-3 if dtype == torch.bfloat16 else 2e-5)
+    assert_state_close(c2, c_r, 2e-5, "C")
+    assert_state_close(n2, n_r, 2e-5, "n")
+    assert (d64(m2) - m_r).abs().max() <= 1e-5
+    if c0_before is not None:
+        assert torch.equal(kw["c_initial"], c0_before), "the initial state must not be modified"
+    # a loop of single steps of the product
+    c = torch.zeros(B, NH, DQK, DHV, device=DEV) if st is None else st[0].to(DEV)
+    n = torch.zeros(B, NH, DQK, device=DEV) if st is None else st[1].to(DEV)
+    m = torch.zeros(B, NH, 1, device=DEV) if st is None else st[2].to(DEV)
+    for t in range(T):
+        h_t, (c, n, m) = step(q[:, :, t].to(DEV), k[:, :, t].to(DEV), v[:, :, t].to(DEV), i[:, :, t, None].to(DEV),
+                              f[:, :, t, None].to(DEV), c, n, m)
+        assert rel_to_scale(H[:, :, t], d64(h_t)) <= (8e-3 if dtype == torch.bfloat16 else 1e-5)
+    assert_state_close(c2, d64(c), 1e-6, "C vs step loop")
+    assert_state_close(n2, d64(n), 1e-6, "n vs step loop")
+
+
+def test_recurrent_sequence_rejects_bad_arguments():
+    from mlstm_kernels_amd import _lib
+    lib = _lib.get_lib()
+    z = torch.zeros(64, device=DEV)
+    p = z.data_ptr()
+    # aliasing n / m, unsupported dtype code, DHQK beyond the register-resident slice, no tokens
+    assert lib.mlstm_hip_recurrent_sequence(p, p, p, p, p, p, p, p, p, p, p, p, 1, 1, 1, 4, 4, 1e-6, 0, 0, None) != 0
+    assert b"alias" in lib.mlstm_hip_last_error()
+    n2, m2 = torch.zeros(64, device=DEV), torch.zeros(64, device=DEV)
+    args = lambda *dims_dt: (p, p, p, p, p, p, p, p, p, p, n2.data_ptr(), m2.data_ptr(), *dims_dt, None)
+    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 1, 4, 4, 1e-6, 7, 0)) != 0
+    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 1, 2048, 4, 1e-6, 0, 0)) != 0
+    assert b"1024" in lib.mlstm_hip_last_error()
+    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 0, 4, 4, 1e-6, 0, 0)) != 0
+
+
 @pytest.mark.parametrize("B", [16, 64, 256])
 def test_decode_after_prefill(B):
     """BASELINE config 5: prefill S=2048 with the chunkwise kernel, then 128 consecutive decode steps (state updated
