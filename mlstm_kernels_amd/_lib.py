@@ -54,6 +54,11 @@ def get_lib() -> ctypes.CDLL:
                     f"{_LIB_PATH} not found. The HIP kernels are the only implementation of this package; "
                     "build them with `python -m mlstm_kernels_amd.build` (needs hipcc, targets gfx950)."
                 )
+            # The host process shares ONE HIP runtime between torch (which owns the device memory and the streams
+            # passed in) and this library: torch is imported first so that its runtime is the one the library binds
+            # to.  Loaded in the other order, two runtimes end up in the process and the second sees no device.
+            import torch  # noqa: F401
+
             lib = ctypes.CDLL(_LIB_PATH)
             for name, (res, args) in _SIGNATURES.items():
                 fn = getattr(lib, name)
