@@ -87,9 +87,13 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   const int n0 = 64 * nh;              // first position (inside the chunk) of this workgroup
   const int stride = a.stride;
   const int slot = c / stride;         // kept boundary state this chunk uses
-  // source chunks of the score blocks: forward c0 .. c (own chunk last), dV c .. c1 (own chunk first)
+  // source chunks of the score blocks: forward c0 .. c, dV c .. c1.  They are walked with the own chunk LAST (forward
+  // upwards, dV downwards): a far chunk's rows are then requested when this workgroup starts, which is when the
+  // workgroups of that chunk -- neighbours in launch order on the same XCD -- request them as their own, so the two
+  // meet in the L2 (walked the other way round, dV fetched 47 % more bytes than it needs).
   const int sc_lo = IS_DV ? c : slot * stride;
   const int sc_hi = IS_DV ? min(slot * stride + stride - 1, NC - 1) : c;
+  const int sc_first = IS_DV ? sc_hi : sc_lo, sc_step = IS_DV ? -1 : 1;
   const uint16_t* Xn_g = (IS_DV ? a.K : a.Q) + (size_t)bh * S * DHQK;
   const uint16_t* Xo_g = (IS_DV ? a.Q : a.K) + (size_t)bh * S * DHQK;
   const uint16_t* Xw_g = (IS_DV ? a.dH : a.V) + (size_t)bh * S * DHHV;
@@ -158,10 +162,10 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         t = {sc, 1, sl_lo + r2, r2 < nv};
       } else {
         r2 -= nv2;
-        t = {sc + 1, 0, r2, sc + 1 <= sc_hi && r2 < nslab};
+        t = {sc + sc_step, 0, r2, sc != c && r2 < nslab};  // the own chunk is the last one
       }
     }
-    if (!t.real) t = {sc_lo, 0, 0, false};
+    if (!t.real) t = {sc_first, 0, 0, false};
     return t;
   };
   // request a slab (and the gate vectors of its source chunk) into register set R_.  A target that is not real makes
@@ -189,8 +193,8 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
       OR_[e] = (IS_DV && a.use_nrow) ? a.nrow[hofs + (size_t)nx_.sc * kChunk + idx_] : 1.f;                          \
     }                                                                                                                \
   }
-  MLSTM_LOAD_AT(sA, ovA, orA, 0, (Target{sc_lo, 0, 0, true}))
-  MLSTM_LOAD_AT(sB, ovB, orB, 0, (Target{sc_lo, 0, nslab > 1 ? 1 : 0, nslab > 1}))
+  MLSTM_LOAD_AT(sA, ovA, orA, 0, (Target{sc_first, 0, 0, true}))
+  MLSTM_LOAD_AT(sB, ovB, orB, 0, (Target{sc_first, 0, nslab > 1 ? 1 : 0, nslab > 1}))
   // state fragments of the first contraction steps of the first column tile: requested up front, together with
   // everything else this workgroup needs first, so that all of it costs ONE trip to memory
   const int m_wave = wave * MW;  // first value column of this wave inside a column tile
@@ -354,8 +358,8 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
           for (int i = 0; i < 16; ++i) acc[tl][mb][nb][i] = 0.f;
     // later groups request their first two slabs only now (the first group's travel since the kernel started)
     if (grp > 0) {
-      MLSTM_LOAD_AT(sA, ovA, orA, grp, (Target{sc_lo, 0, 0, true}))
-      MLSTM_LOAD_AT(sB, ovB, orB, grp, (Target{sc_lo, 0, nslab > 1 ? 1 : 0, nslab > 1}))
+      MLSTM_LOAD_AT(sA, ovA, orA, grp, (Target{sc_first, 0, 0, true}))
+      MLSTM_LOAD_AT(sB, ovB, orB, grp, (Target{sc_first, 0, nslab > 1 ? 1 : 0, nslab > 1}))
     }
     __syncthreads();  // phase-0 writes visible (later groups: the previous group's output staging is stored)
     // ---- inter-chunk product, tile by tile: Out^T = State^T Xn^T
@@ -403,7 +407,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
     }
 
     // ---- source chunks: score block, gated into Ps, then Out^T += Xw^T P for every value column of the group
-    for (int sc = sc_lo; sc <= sc_hi; ++sc) {
+    for (int sc = sc_first; sc >= sc_lo && sc <= sc_hi; sc += sc_step) {
       int ob_lo, ob_hi;
       ob_range(sc, ob_lo, ob_hi);
       int sl_lo, sl_hi;
