@@ -390,7 +390,8 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     dict(B=1, NH=2, S=256, DQK=64, DHV=128),
     dict(B=2, NH=2, S=512, DQK=128, DHV=256, seed=1),
     dict(B=1, NH=2, S=384, DQK=256, DHV=512, init=True, dcl=True),
-    dict(B=1, NH=1, S=256, DQK=512, DHV=256, init=True),          # two head-dim tiles: atomic row dots
+    dict(B=1, NH=1, S=256, DQK=512, DHV=256, init=True),          # two head-dim tiles: one row-dot slot each
+    dict(B=1, NH=1, S=384, DQK=896, DHV=128, init=True, seed=7),  # the largest head dimension the resident tile holds
     dict(B=1, NH=2, S=256, DQK=64, DHV=128, siging=True, init=True),
     dict(B=1, NH=2, S=256, DQK=64, DHV=64, siging=True, normalize=False),
     dict(B=1, NH=2, S=144, DQK=64, DHV=64, L=16),                  # ragged tail
