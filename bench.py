@@ -372,8 +372,36 @@ def main():
                 "tokens_per_s": round(Bd * T / (ms * 1e-3), 1),
                 "state_bytes_moved": 2 * Bd * NH * DHQK * DHHV * 4}
 
+    # ---- the step with its states kept in bfloat16 (half the bytes per step; arithmetic still fp32)
+    def bench_decode_bf16_state(Bd):
+        bf = torch.bfloat16
+        c, n, m = rn(Bd, NH, DHQK, DHHV).to(bf), rn(Bd, NH, DHQK).to(bf), rn(Bd, NH, 1).to(bf)
+        n_alt, m_alt = torch.empty_like(n), torch.empty_like(m)
+        total = DECODE_WARMUP + DECODE_STEPS
+        qs, ks, vs = rn(total, Bd, NH, DHQK).to(bf), rn(total, Bd, NH, DHQK).to(bf), rn(total, Bd, NH, DHHV).to(bf)
+        is_, fs = rn(total, Bd, NH, 1), 3 + rn(total, Bd, NH, 1)
+        _lib.profile_read()
+        for t in range(total):
+            if t == DECODE_WARMUP:
+                torch.cuda.synchronize()
+                _lib.profile_enable(True)
+                t0 = time.perf_counter()
+            _, (c, n_new, m_new) = mlstm_recurrent_step__hip_fw(c, n, m, qs[t], ks[t], vs[t], is_[t], fs[t], matC_new=c,
+                                                               vecN_new=n_alt, scaM_new=m_alt, dtype_state=bf)
+            n_alt, m_alt, n, m = n, m, n_new, m_new
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / DECODE_STEPS * 1e3
+        _lib.profile_enable(False)
+        st_ms, st_cnt = _lib.profile_read().get("step", (0.0, 1))
+        nbytes = (2 * DHQK * DHHV * 2 + 2 * DHQK * 2 + 2 * 2 + (2 * DHQK + DHHV) * 2 + DHHV * 2 + 2 * 4) * Bd * NH
+        return {"batch": Bd, "mode": "eager, bfloat16 states", "steps": DECODE_STEPS, "ms_per_step": round(ms, 4),
+                "kernel_ms": round(st_ms / max(st_cnt, 1), 4), "bytes_per_step": nbytes,
+                "value": round(nbytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                "bound": "hbm" if c.numel() * 2 > MALL_BYTES else "mall"}
+
     decode = bench_decode(DECODE_B, graph=False)
     if not args.no_extra:
+        decode["bf16_state"] = bench_decode_bf16_state(DECODE_B)
         decode["other_batches"] = [bench_decode(b, graph=g_) for b in (64, 16) for g_ in (False, True)]
         decode["multi_token"] = [bench_decode_sequence(b) for b in (DECODE_B, 64, 16)]
     torch.cuda.empty_cache()

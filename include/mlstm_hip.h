@@ -92,14 +92,17 @@ const char* mlstm_hip_last_error(void);
  * Replaces: mlstm_kernels/torch/recurrent/triton_step.py:15-127 (mlstm_recurrent_step__triton_fw) and the
  * Triton kernel mlstm_kernels/triton/recurrent/fw_step_fused.py:19-195.
  *   q,k (B,NH,DHQK), v (B,NH,DHHV) in dtype_qkv; i,f (B,NH) in dtype_gates; h (B,NH,DHHV) in dtype_qkv.
+ *   States C (B,NH,DHQK,DHHV), n (B,NH,DHQK), m (B,NH) in and out in dtype_state (MLSTM_F32 or MLSTM_BF16: the
+ *   reference's dtype_state, triton_step.py:33,67-69); the arithmetic is fp32 either way, h is formed from the
+ *   unrounded new state.  DHHV % 4 == 0 (fp32 state) or % 8 == 0 (bf16 state).
  *   c_out may alias c_in (in-place update of the state matrix); n_out/m_out must be distinct from n_in/m_in
  *   (every workgroup of a head reads the old n and m while one of them writes the new values).
  */
 int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f,
-                   const float* c_in, const float* n_in, const float* m_in,
-                   void* h, float* c_out, float* n_out, float* m_out,
+                   const void* c_in, const void* n_in, const void* m_in,
+                   void* h, void* c_out, void* n_out, void* m_out,
                    int B, int NH, int DHQK, int DHHV, float eps,
-                   int dtype_qkv, int dtype_gates, void* stream);
+                   int dtype_qkv, int dtype_gates, int dtype_state, void* stream);
 
 /*
  * Recurrent mLSTM over T tokens in one launch (multi-token decode, the remainder of a prefill): the step above
@@ -108,14 +111,15 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
  * Replaces: the token loop mlstm_kernels/torch/recurrent/native_sequence.py:13-122
  * (mlstm_recurrent_sequence__triton_step_fused_fw = _mlstm_recurrent_sequence_loop_fw over the fused step).
  *   q,k (B,NH,T,DHQK), v (B,NH,T,DHHV) in dtype_qkv; i,f (B,NH,T) in dtype_gates; h (B,NH,T,DHHV) in dtype_qkv;
- *   states as for mlstm_hip_step (c_out may alias c_in, n_out/m_out must be distinct from n_in/m_in).
+ *   states as for mlstm_hip_step (dtype_state; between tokens the state stays fp32 in registers, so a bf16 state is
+ *   rounded once per call, not once per token; c_out may alias c_in, n_out/m_out must be distinct from n_in/m_in).
  *   DHQK <= 1024.
  */
 int mlstm_hip_recurrent_sequence(const void* q, const void* k, const void* v, const void* i, const void* f,
-                                 const float* c_in, const float* n_in, const float* m_in,
-                                 void* h, float* c_out, float* n_out, float* m_out,
+                                 const void* c_in, const void* n_in, const void* m_in,
+                                 void* h, void* c_out, void* n_out, void* m_out,
                                  int B, int NH, int T, int DHQK, int DHHV, float eps,
-                                 int dtype_qkv, int dtype_gates, void* stream);
+                                 int dtype_qkv, int dtype_gates, int dtype_state, void* stream);
 
 /*
  * Bytes of caller-provided workspace the chunkwise forward needs.  With keep_for_backward != 0 the

@@ -13,7 +13,7 @@ F32, BF16 = 0, 1
 GATE_EXP, GATE_SIG = 0, 1
 PATH_AUTO, PATH_SPLIT, PATH_FUSED = 0, 1, 2
 NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2
-ABI_VERSION = 4
+ABI_VERSION = 5
 NOALLOC_SCRATCH_BYTES = 64 << 20  # MLSTM_NOALLOC_SCRATCH_BYTES of include/mlstm_hip.h
 
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
@@ -23,8 +23,8 @@ _SIGNATURES = {
     "mlstm_hip_last_error": (ctypes.c_char_p, []),
     "mlstm_hip_profile_enable": (_i, [_i]),
     "mlstm_hip_profile_read": (_i, [_i, ctypes.c_char_p, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_int)]),
-    "mlstm_hip_step": (_i, [_vp] * 12 + [_i, _i, _i, _i, _f, _i, _i, _vp]),
-    "mlstm_hip_recurrent_sequence": (_i, [_vp] * 12 + [_i, _i, _i, _i, _i, _f, _i, _i, _vp]),
+    "mlstm_hip_step": (_i, [_vp] * 12 + [_i, _i, _i, _i, _f, _i, _i, _i, _vp]),
+    "mlstm_hip_recurrent_sequence": (_i, [_vp] * 12 + [_i, _i, _i, _i, _i, _f, _i, _i, _i, _vp]),
     "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 8),
     "mlstm_hip_chunkwise_fw": (_i, [_vp] * 15 + [_sz, _i] + [_i] * 5 + [_f] + [_i] * 7 + [_f, _vp, _vp] + [_vp]),
     "mlstm_hip_head_norm_bw": (_i, [_vp] * 4 + [_sz, _i, _i, _i, _vp]),

@@ -92,7 +92,7 @@ int set_last_error(const char* msg) { return fail(msg); }
 
 extern "C" {
 
-int mlstm_hip_abi_version(void) { return 4; }
+int mlstm_hip_abi_version(void) { return 5; }
 
 int mlstm_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
@@ -132,38 +132,40 @@ int mlstm_hip_profile_read(int index, char* name, size_t name_cap, float* total_
 }
 const char* mlstm_hip_last_error(void) { return g_err; }
 
-int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f, const float* c_in,
-                   const float* n_in, const float* m_in, void* h, float* c_out, float* n_out, float* m_out, int B,
-                   int NH, int DHQK, int DHHV, float eps, int dtype_qkv, int dtype_gates, void* stream) {
+int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, const void* f, const void* c_in,
+                   const void* n_in, const void* m_in, void* h, void* c_out, void* n_out, void* m_out, int B, int NH,
+                   int DHQK, int DHHV, float eps, int dtype_qkv, int dtype_gates, int dtype_state, void* stream) {
   if (!q || !k || !v || !i || !f || !c_in || !n_in || !m_in || !h || !c_out || !n_out || !m_out)
     return fail("mlstm_hip_step: null pointer argument");
   if (n_out == n_in || m_out == m_in)
     return fail("mlstm_hip_step: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
-  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16))
+  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) ||
+      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16))
     return fail("mlstm_hip_step: unsupported dtype code");
   {
     ProfileScope ps("step", (hipStream_t)stream);
     const char* e = mlstm::launch_step(q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps,
-                                       dtype_qkv, dtype_gates, (hipStream_t)stream);
+                                       dtype_qkv, dtype_gates, dtype_state, (hipStream_t)stream);
     if (e) return fail(e);
   }
   return check_launch("mlstm_hip_step");
 }
 
 int mlstm_hip_recurrent_sequence(const void* q, const void* k, const void* v, const void* i, const void* f,
-                                 const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                                 float* n_out, float* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
-                                 int dtype_qkv, int dtype_gates, void* stream) {
+                                 const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                                 void* n_out, void* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
+                                 int dtype_qkv, int dtype_gates, int dtype_state, void* stream) {
   if (!q || !k || !v || !i || !f || !c_in || !n_in || !m_in || !h || !c_out || !n_out || !m_out)
     return fail("mlstm_hip_recurrent_sequence: null pointer argument");
   if (n_out == n_in || m_out == m_in)
     return fail("mlstm_hip_recurrent_sequence: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
-  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16))
+  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) ||
+      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16))
     return fail("mlstm_hip_recurrent_sequence: unsupported dtype code");
   {
     ProfileScope ps("step_seq", (hipStream_t)stream);
     const char* e = mlstm::launch_step_seq(q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, T, DHQK, DHHV,
-                                           eps, dtype_qkv, dtype_gates, (hipStream_t)stream);
+                                           eps, dtype_qkv, dtype_gates, dtype_state, (hipStream_t)stream);
     if (e) return fail(e);
   }
   return check_launch("mlstm_hip_recurrent_sequence");

@@ -102,13 +102,13 @@ struct GateGradArgs {
 };
 
 const char* launch_step(const void* q, const void* k, const void* v, const void* i, const void* f,
-                        const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                        float* n_out, float* m_out, int B, int NH, int DHQK, int DHHV, float eps,
-                        int dtype_qkv, int dtype_gates, hipStream_t stream);
+                        const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                        void* n_out, void* m_out, int B, int NH, int DHQK, int DHHV, float eps,
+                        int dtype_qkv, int dtype_gates, int dtype_state, hipStream_t stream);
 const char* launch_step_seq(const void* q, const void* k, const void* v, const void* i, const void* f,
-                            const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                            float* n_out, float* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
-                            int dtype_qkv, int dtype_gates, hipStream_t stream);
+                            const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                            void* n_out, void* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
+                            int dtype_qkv, int dtype_gates, int dtype_state, hipStream_t stream);
 const char* launch_gates(const void* i, const void* f, const float* m0, const GateBufs& gb, float* m_last,
                          int B, int NH, int S, int dtype_gates, int sig_gate, hipStream_t stream);
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream);

@@ -6,9 +6,10 @@
 //
 // (math of mlstm_kernels/torch/recurrent/native_step.py:69-95 in the reference; everything in fp32.)
 //
-// The step is a pure stream over the fp32 state C (DHQK x DHHV per head): one read and one write of every
-// element, 0.75 flop per byte, so it is laid out for HBM bandwidth only -- no matrix cores.  A workgroup
-// owns (b, head, slice of COLS value columns); COLS/4 lanes x 16 B cover one contiguous row segment and the TY
+// The step is a pure stream over the state C (DHQK x DHHV per head; fp32, or bfloat16 when the caller keeps its states
+// in that type): one read and one write of every element, 0.75 flop per byte at fp32, so it is laid out for HBM
+// bandwidth only -- no matrix cores.  A workgroup owns (b, head, slice of COLS value columns); lanes of 16 B (four fp32
+// or eight bf16 columns) cover one contiguous row segment and the TY
 // row groups of the workgroup walk the DHQK rows with all loads of an unrolled batch in flight before the first
 // use.  The q^T C' column sums are reduced across the row groups through LDS at the end.
 #include "common.h"
@@ -16,15 +17,59 @@
 
 namespace mlstm {
 
-template <int COLS, int TY, int UNROLL, bool NONTEMPORAL>
-__global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
+// One 16-byte piece of a state row: four fp32 columns, or eight bf16 columns when the state is kept in bfloat16
+// (the reference's dtype_state / inference_state_dtype, mlstm_kernels/torch/recurrent/triton_step.py:33,67-69).
+template <bool SBF>
+struct StatePiece {
+  static constexpr int N = SBF ? 8 : 4;
+  float x[N];
+};
+template <bool SBF, bool NT>
+__device__ __forceinline__ StatePiece<SBF> load_piece(const void* base, size_t elem) {
+  StatePiece<SBF> p;
+  if constexpr (SBF) {
+    const u32x4* src = (const u32x4*)((const uint16_t*)base + elem);
+    const u32x4 raw = NT ? __builtin_nontemporal_load(src) : *src;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      p.x[2 * e] = __uint_as_float(raw[e] << 16);
+      p.x[2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
+    }
+  } else {
+    const f32x4* src = (const f32x4*)((const float*)base + elem);
+    const f32x4 raw = NT ? __builtin_nontemporal_load(src) : *src;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) p.x[e] = raw[e];
+  }
+  return p;
+}
+template <bool SBF, bool NT>
+__device__ __forceinline__ void store_piece(void* base, size_t elem, const StatePiece<SBF>& p) {
+  if constexpr (SBF) {
+    const u32x4 raw = {pack_bf16x2(p.x[0], p.x[1]), pack_bf16x2(p.x[2], p.x[3]), pack_bf16x2(p.x[4], p.x[5]),
+                       pack_bf16x2(p.x[6], p.x[7])};
+    u32x4* dst = (u32x4*)((uint16_t*)base + elem);
+    if (NT) __builtin_nontemporal_store(raw, dst);
+    else *dst = raw;
+  } else {
+    const f32x4 raw = {p.x[0], p.x[1], p.x[2], p.x[3]};
+    f32x4* dst = (f32x4*)((float*)base + elem);
+    if (NT) __builtin_nontemporal_store(raw, dst);
+    else *dst = raw;
+  }
+}
+
+template <int COLS, int TY, int UNROLL, bool NONTEMPORAL, bool SBF>
+__global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
     const void* __restrict__ ig, const void* __restrict__ fg,
-    const float* c_in, const float* n_in, const float* m_in,
-    void* __restrict__ h, float* c_out, float* n_out, float* m_out,
+    const void* c_in, const void* n_in, const void* m_in,
+    void* __restrict__ h, void* c_out, void* n_out, void* m_out,
     int DHQK, int DHHV, float eps, int dtype_qkv, int dtype_gates) {
-  constexpr int TX = COLS / 4;
+  constexpr int VPL = StatePiece<SBF>::N;   // state columns per lane
+  constexpr int TX = COLS / VPL;
   constexpr int NTH = TX * TY;
+  constexpr int dtype_state = SBF ? 1 : 0;
   extern __shared__ float smem[];
   float* qs = smem;                 // [DHQK] q / sqrt(d)
   float* ik = smem + DHQK;          // [DHQK] i' * k
@@ -39,22 +84,24 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
   // and the LDS staging below are computed (none of which they depend on).  With a large state many workgroups
   // per CU overlap each other's prologues and the extra live registers only cost occupancy (measured: 0.373 ms
   // against 0.358 ms at B = 256), so the streaming variant does not do it.
-  const int col = col0 + 4 * tx;
-  const bool col_ok = col < DHHV;  // DHHV % 4 == 0 is checked on the host
-  const float* cin = c_in + (size_t)bh * DHQK * DHHV + col;
-  float* cout = c_out + (size_t)bh * DHQK * DHHV + col;
+  const int col = col0 + VPL * tx;
+  const bool col_ok = col < DHHV;  // DHHV % VPL == 0 is checked on the host
+  const size_t cbase = (size_t)bh * DHQK * DHHV + col;
   const bool have_first = !NONTEMPORAL && col_ok && ty + (UNROLL - 1) * TY < DHQK;
-  f32x4 cfirst[UNROLL];
+  StatePiece<SBF> cfirst[UNROLL];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-    const f32x4* p = (const f32x4*)(cin + (size_t)(ty + u * TY) * DHHV);
-    cfirst[u] = have_first ? *p : z;
+    if (have_first) {
+      cfirst[u] = load_piece<SBF, false>(c_in, cbase + (size_t)(ty + u * TY) * DHHV);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VPL; ++e) cfirst[u].x[e] = 0.f;
+    }
   }
 
   const float fpre = load_scalar(fg, bh, dtype_gates);
   const float ipre = load_scalar(ig, bh, dtype_gates);
-  const float m_old = m_in[bh];
+  const float m_old = load_scalar(m_in, bh, dtype_state);
   const float lf = log_sigmoid(fpre);
   const float m_new = fmaxf(lf + m_old, ipre);
   const float fa = expf(lf + m_old - m_new);
@@ -67,11 +114,14 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
     const size_t o = (size_t)bh * DHQK + d;
     const float qd = load_scalar(q, o, dtype_qkv) * scale;
     const float kd = load_scalar(k, o, dtype_qkv);
-    const float nd = fa * n_in[o] + ia * kd;
+    const float nd = fa * load_scalar(n_in, o, dtype_state) + ia * kd;
     qs[d] = qd;
     ik[d] = ia * kd;
     qn_part += qd * nd;
-    if (blockIdx.x == 0) n_out[o] = nd;
+    if (blockIdx.x == 0) {
+      if (SBF) ((uint16_t*)n_out)[o] = f32_to_bf16_bits(nd);
+      else ((float*)n_out)[o] = nd;
+    }
   }
   qn_part = wave_sum(qn_part);
   __shared__ float wsum[(NTH + kWave - 1) / kWave];
@@ -81,59 +131,75 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
 #pragma unroll
   for (int w = 0; w < (NTH + kWave - 1) / kWave; ++w) qn += wsum[w];
   const float inv_den = 1.f / (fmaxf(fabsf(qn), expf(-m_new)) + eps);
-  if (blockIdx.x == 0 && tid == 0) m_out[bh] = m_new;
+  if (blockIdx.x == 0 && tid == 0) {
+    if (SBF) ((uint16_t*)m_out)[bh] = f32_to_bf16_bits(m_new);
+    else ((float*)m_out)[bh] = m_new;
+  }
 
-  f32x4 v4 = {0.f, 0.f, 0.f, 0.f};
+  float vv[VPL];
+#pragma unroll
+  for (int e = 0; e < VPL; ++e) vv[e] = 0.f;
   if (col_ok) {
     const size_t o = (size_t)bh * DHHV + col;
     if (dtype_qkv == 0) {
-      v4 = *(const f32x4*)((const float*)v + o);
+#pragma unroll
+      for (int e4 = 0; e4 < VPL / 4; ++e4) {
+        const f32x4 raw = *(const f32x4*)((const float*)v + o + 4 * e4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vv[4 * e4 + e] = raw[e];
+      }
     } else {
-      const uint2 raw = *(const uint2*)((const uint16_t*)v + o);
-      v4[0] = __uint_as_float(raw.x << 16);
-      v4[1] = __uint_as_float(raw.x & 0xffff0000u);
-      v4[2] = __uint_as_float(raw.y << 16);
-      v4[3] = __uint_as_float(raw.y & 0xffff0000u);
+#pragma unroll
+      for (int e4 = 0; e4 < VPL / 4; ++e4) {
+        const uint2 raw = *(const uint2*)((const uint16_t*)v + o + 4 * e4);
+        vv[4 * e4 + 0] = __uint_as_float(raw.x << 16);
+        vv[4 * e4 + 1] = __uint_as_float(raw.x & 0xffff0000u);
+        vv[4 * e4 + 2] = __uint_as_float(raw.y << 16);
+        vv[4 * e4 + 3] = __uint_as_float(raw.y & 0xffff0000u);
+      }
     }
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float acc[VPL];
+#pragma unroll
+  for (int e = 0; e < VPL; ++e) acc[e] = 0.f;
+  // C' = f' C + i' k v^T for one piece of row rr; q^T C' accumulates from the fp32 values (before any rounding)
+  auto update = [&](const StatePiece<SBF>& cold, int rr) {
+    StatePiece<SBF> o;
+    const float ikr = ik[rr], qr = qs[rr];
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) {
+      o.x[e] = fa * cold.x[e] + ikr * vv[e];
+      acc[e] += qr * o.x[e];
+    }
+    return o;
+  };
   if (col_ok) {
     int r = ty;
     if (have_first) {
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const int rr = r + u * TY;
-        const f32x4 o = fa * cfirst[u] + ik[rr] * v4;
-        *(f32x4*)(cout + (size_t)rr * DHHV) = o;
-        acc += qs[rr] * o;
+        store_piece<SBF, false>(c_out, cbase + (size_t)rr * DHHV, update(cfirst[u], rr));
       }
       r += UNROLL * TY;
     }
     for (; r + (UNROLL - 1) * TY < DHQK; r += UNROLL * TY) {
-      f32x4 c[UNROLL];
+      StatePiece<SBF> c[UNROLL];
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const f32x4* p = (const f32x4*)(cin + (size_t)(r + u * TY) * DHHV);
-        c[u] = NONTEMPORAL ? __builtin_nontemporal_load(p) : *p;
-      }
+      for (int u = 0; u < UNROLL; ++u) c[u] = load_piece<SBF, NONTEMPORAL>(c_in, cbase + (size_t)(r + u * TY) * DHHV);
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const int rr = r + u * TY;
-        const f32x4 o = fa * c[u] + ik[rr] * v4;
-        f32x4* p = (f32x4*)(cout + (size_t)rr * DHHV);
-        if (NONTEMPORAL) __builtin_nontemporal_store(o, p);
-        else *p = o;
-        acc += qs[rr] * o;
+        store_piece<SBF, NONTEMPORAL>(c_out, cbase + (size_t)rr * DHHV, update(c[u], rr));
       }
     }
     for (; r < DHQK; r += TY) {
-      const f32x4 c = *(const f32x4*)(cin + (size_t)r * DHHV);
-      const f32x4 o = fa * c + ik[r] * v4;
-      *(f32x4*)(cout + (size_t)r * DHHV) = o;
-      acc += qs[r] * o;
+      const StatePiece<SBF> c = load_piece<SBF, false>(c_in, cbase + (size_t)r * DHHV);
+      store_piece<SBF, false>(c_out, cbase + (size_t)r * DHHV, update(c, r));
     }
   }
-  *(f32x4*)(red + ty * COLS + 4 * tx) = acc;
+#pragma unroll
+  for (int e = 0; e < VPL; ++e) red[ty * COLS + VPL * tx + e] = acc[e];
   __syncthreads();
   for (int cidx = tid; cidx < COLS; cidx += NTH) {
     if (col0 + cidx < DHHV) {
@@ -148,44 +214,46 @@ __global__ __launch_bounds__((COLS / 4) * TY) void step_kernel(
   }
 }
 
-template <int COLS, int TY, int UNROLL, bool NONTEMPORAL>
+template <int COLS, int TY, int UNROLL, bool NONTEMPORAL, bool SBF>
 static const char* launch_step_t(const void* q, const void* k, const void* v, const void* i, const void* f,
-                                 const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                                 float* n_out, float* m_out, int B, int NH, int DHQK, int DHHV, float eps,
+                                 const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                                 void* n_out, void* m_out, int B, int NH, int DHQK, int DHHV, float eps,
                                  int dtype_qkv, int dtype_gates, hipStream_t stream) {
   const size_t smem = (size_t)(2 * DHQK + TY * COLS) * sizeof(float);
   if (smem > 64 * 1024) return "mlstm_hip_step: DHQK too large for the LDS staging";
   dim3 grid((DHHV + COLS - 1) / COLS, B * NH);
-  hipLaunchKernelGGL((step_kernel<COLS, TY, UNROLL, NONTEMPORAL>), grid, dim3((COLS / 4) * TY), smem, stream, q, k, v,
-                     i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, DHQK, DHHV, eps, dtype_qkv, dtype_gates);
+  hipLaunchKernelGGL((step_kernel<COLS, TY, UNROLL, NONTEMPORAL, SBF>), grid, dim3((COLS / StatePiece<SBF>::N) * TY), smem,
+                     stream, q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, DHQK, DHHV, eps, dtype_qkv,
+                     dtype_gates);
   return nullptr;
 }
 
-#ifndef MLSTM_STEP_NO_DEFAULT_LAUNCHER
 const char* launch_step(const void* q, const void* k, const void* v, const void* i, const void* f,
-                        const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                        float* n_out, float* m_out, int B, int NH, int DHQK, int DHHV, float eps,
-                        int dtype_qkv, int dtype_gates, hipStream_t stream) {
+                        const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                        void* n_out, void* m_out, int B, int NH, int DHQK, int DHHV, float eps,
+                        int dtype_qkv, int dtype_gates, int dtype_state, hipStream_t stream) {
   if (B <= 0 || NH <= 0 || DHQK <= 0 || DHHV <= 0) return "mlstm_hip_step: non-positive dimension";
-  if (DHHV % 4 != 0) return "mlstm_hip_step: DHHV must be a multiple of 4";
+  const bool sbf = dtype_state != 0;
+  if (DHHV % (sbf ? 8 : 4) != 0)
+    return sbf ? "mlstm_hip_step: DHHV must be a multiple of 8 for a bfloat16 state" : "mlstm_hip_step: DHHV must be a multiple of 4";
   if ((long long)B * NH > 65535) return "mlstm_hip_step: B*NH exceeds 65535";
-  // Tile shapes from a sweep on MI355X (B = 16/64/256, NH = 8, 256 x 512 state).  A state larger than the 256 MB
+  // Tile shapes from a sweep on MI355X (B = 16/64/256, NH = 8, 256 x 512 fp32 state).  A state larger than the 256 MB
   // memory-side cache streams past the caches with non-temporal accesses: 256-column slices, 8 row groups, 16 rows
   // in flight per lane.  A smaller one is best left cacheable (it is re-read by the next step) and has few
   // workgroups per CU: 128-column slices with 16 row groups, the first 16 rows per lane requested before the
   // prologue.  The crossover was measured between a 268 MB state (cacheable 79 us, streaming 90 us) and a 403 MB
-  // state (156 us against 133 us).
-  const size_t state_bytes = (size_t)B * NH * DHQK * DHHV * sizeof(float);
+  // state (156 us against 133 us).  A bfloat16 state uses the same shapes with lanes of eight columns (half as many
+  // lanes per row segment), so every lane still moves 16 bytes per access.
+  const size_t state_bytes = (size_t)B * NH * DHQK * DHHV * (sbf ? 2 : 4);
   const bool stream_past_cache = state_bytes > ((size_t)320 << 20);
 #define MLSTM_STEP_ARGS q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps, dtype_qkv, dtype_gates, stream
-  if (DHHV % 256 == 0) {
-    if (stream_past_cache) return launch_step_t<256, 8, 16, true>(MLSTM_STEP_ARGS);
-    return launch_step_t<128, 16, 16, false>(MLSTM_STEP_ARGS);
-  }
-  if (stream_past_cache) return launch_step_t<128, 8, 8, true>(MLSTM_STEP_ARGS);
-  return launch_step_t<128, 16, 16, false>(MLSTM_STEP_ARGS);
+#define MLSTM_STEP_PICK(COLS_, TY_, UN_, NT_) \
+  return sbf ? launch_step_t<COLS_, TY_, UN_, NT_, true>(MLSTM_STEP_ARGS) : launch_step_t<COLS_, TY_, UN_, NT_, false>(MLSTM_STEP_ARGS)
+  if (DHHV % 256 == 0 && stream_past_cache) MLSTM_STEP_PICK(256, 8, 16, true);
+  if (stream_past_cache) MLSTM_STEP_PICK(128, 8, 8, true);
+  MLSTM_STEP_PICK(128, 16, 16, false);
+#undef MLSTM_STEP_PICK
 #undef MLSTM_STEP_ARGS
 }
-#endif
 
 }  // namespace mlstm

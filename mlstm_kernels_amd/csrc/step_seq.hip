@@ -48,9 +48,9 @@ __global__ __launch_bounds__(64)
     __attribute__((amdgpu_waves_per_eu(STEP_SEQ_WPE(RPT * CPT), STEP_SEQ_WPE(RPT * CPT)))) void step_seq_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
     const void* __restrict__ ig, const void* __restrict__ fg,
-    const float* c_in, const float* n_in, const float* m_in,
-    void* __restrict__ h, float* c_out, float* n_out, float* m_out,
-    int T, int DHQK, int DHHV, float eps, int dtype_gates) {
+    const void* c_in, const void* n_in, const void* m_in,
+    void* __restrict__ h, void* c_out, void* n_out, void* m_out,
+    int T, int DHQK, int DHHV, float eps, int dtype_gates, int dtype_state) {
   constexpr int NG = 8;                       // row groups per column (neighbouring lanes)
   constexpr int COLS = 8 * CPT;               // value columns per workgroup
   constexpr int DMAX = RPT * NG;              // largest DHQK this instantiation holds
@@ -78,18 +78,30 @@ __global__ __launch_bounds__(64)
   // (loads are unconditional from clamped addresses, the result is selected afterwards: no branches around them)
   float C[RPT][CPT];
   const bool col_in = col < DHHV;
+  const bool sbf = dtype_state != 0;  // states in and out in bfloat16 (fp32 in registers between the tokens)
 #pragma unroll
   for (int u = 0; u < RPT; ++u) {
     const int r = g * RPT + u;
-    const float* src = c_in + ((size_t)bh * DHQK + min(r, DHQK - 1)) * DHHV;
+    const size_t row = ((size_t)bh * DHQK + min(r, DHQK - 1)) * DHHV;
     if constexpr (VEC) {
-      const f32x4 x = *(const f32x4*)(src + (col_in ? col : 0));
+      float x[4];
+      if (sbf) {
+        const uint2 raw = *(const uint2*)((const uint16_t*)c_in + row + (col_in ? col : 0));
+        x[0] = __uint_as_float(raw.x << 16);
+        x[1] = __uint_as_float(raw.x & 0xffff0000u);
+        x[2] = __uint_as_float(raw.y << 16);
+        x[3] = __uint_as_float(raw.y & 0xffff0000u);
+      } else {
+        const f32x4 raw = *(const f32x4*)((const float*)c_in + row + (col_in ? col : 0));
 #pragma unroll
-      for (int e = 0; e < CPT; ++e) C[u][e] = (r < DHQK && col_in) ? x[e] : 0.f;
+        for (int e = 0; e < 4; ++e) x[e] = raw[e];
+      }
+#pragma unroll
+      for (int e = 0; e < CPT; ++e) C[u][e] = (r < DHQK && col_in) ? x[e & 3] : 0.f;
     } else {
 #pragma unroll
       for (int e = 0; e < CPT; ++e) {
-        const float x = src[min(col + e, DHHV - 1)];
+        const float x = load_scalar(c_in, row + min(col + e, DHHV - 1), dtype_state);
         C[u][e] = (r < DHQK && col + e < DHHV) ? x : 0.f;
       }
     }
@@ -98,13 +110,13 @@ __global__ __launch_bounds__(64)
 #pragma unroll
   for (int j = 0; j < NDJ; ++j) {
     const int d = lane + j * kWave;
-    nreg[j] = d < DHQK ? n_in[(size_t)bh * DHQK + d] : 0.f;
+    nreg[j] = d < DHQK ? load_scalar(n_in, (size_t)bh * DHQK + d, dtype_state) : 0.f;
   }
   for (int x = lane; x < 2 * NG * RS; x += kWave) {
     (&qs[0][0])[x] = 0.f;
     (&ik[0][0])[x] = 0.f;
   }
-  float m = m_in[bh];
+  float m = load_scalar(m_in, bh, dtype_state);
 
   // ---- token inputs, PF tokens ahead, in a ring that is shifted by one slot per token.  Tokens past the end
   // re-request the last one (nobody uses them): an unconditional load keeps the ring in registers.
@@ -301,16 +313,24 @@ __global__ __launch_bounds__(64)
   for (int u = 0; u < RPT; ++u) {
     const int r = g * RPT + u;
     if (r < DHQK) {
-      float* dst = c_out + ((size_t)bh * DHQK + r) * DHHV;
+      const size_t row = ((size_t)bh * DHQK + r) * DHHV;
       if constexpr (vec_ok) {
         if (col_in) {
-          const f32x4 y = {C[u][0], C[u][1 % CPT], C[u][2 % CPT], C[u][3 % CPT]};
-          *(f32x4*)(dst + col) = y;
+          if (sbf) {
+            *(uint2*)((uint16_t*)c_out + row + col) =
+                make_uint2(pack_bf16x2(C[u][0], C[u][1 % CPT]), pack_bf16x2(C[u][2 % CPT], C[u][3 % CPT]));
+          } else {
+            const f32x4 y = {C[u][0], C[u][1 % CPT], C[u][2 % CPT], C[u][3 % CPT]};
+            *(f32x4*)((float*)c_out + row + col) = y;
+          }
         }
       } else {
 #pragma unroll
         for (int e = 0; e < CPT; ++e)
-          if (col + e < DHHV) dst[col + e] = C[u][e];
+          if (col + e < DHHV) {
+            if (sbf) ((uint16_t*)c_out)[row + col + e] = f32_to_bf16_bits(C[u][e]);
+            else ((float*)c_out)[row + col + e] = C[u][e];
+          }
       }
     }
   }
@@ -318,32 +338,38 @@ __global__ __launch_bounds__(64)
 #pragma unroll
     for (int j = 0; j < NDJ; ++j) {
       const int d = lane + j * kWave;
-      if (d < DHQK) n_out[(size_t)bh * DHQK + d] = nreg[j];
+      if (d < DHQK) {
+        if (sbf) ((uint16_t*)n_out)[(size_t)bh * DHQK + d] = f32_to_bf16_bits(nreg[j]);
+        else ((float*)n_out)[(size_t)bh * DHQK + d] = nreg[j];
+      }
     }
-    if (lane == 0) m_out[bh] = m;
+    if (lane == 0) {
+      if (sbf) ((uint16_t*)m_out)[bh] = f32_to_bf16_bits(m);
+      else ((float*)m_out)[bh] = m;
+    }
   }
 }
 
 template <int RPT, int CPT, bool VEC, bool BF16>
 static const char* launch_step_seq_t(const void* q, const void* k, const void* v, const void* i, const void* f,
-                                     const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                                     float* n_out, float* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
-                                     int dtype_qkv, int dtype_gates, hipStream_t stream) {
+                                     const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                                     void* n_out, void* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
+                                     int dtype_qkv, int dtype_gates, int dtype_state, hipStream_t stream) {
   constexpr int COLS = 8 * CPT;
   dim3 grid((DHHV + COLS - 1) / COLS, B * NH);
   hipLaunchKernelGGL((step_seq_kernel<RPT, CPT, VEC, BF16>), grid, dim3(64), 0, stream, q, k, v, i, f, c_in, n_in, m_in, h,
-                     c_out, n_out, m_out, T, DHQK, DHHV, eps, dtype_gates);
+                     c_out, n_out, m_out, T, DHQK, DHHV, eps, dtype_gates, dtype_state);
   return nullptr;
 }
 
 const char* launch_step_seq(const void* q, const void* k, const void* v, const void* i, const void* f,
-                            const float* c_in, const float* n_in, const float* m_in, void* h, float* c_out,
-                            float* n_out, float* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
-                            int dtype_qkv, int dtype_gates, hipStream_t stream) {
+                            const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
+                            void* n_out, void* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
+                            int dtype_qkv, int dtype_gates, int dtype_state, hipStream_t stream) {
   if (B <= 0 || NH <= 0 || T <= 0 || DHQK <= 0 || DHHV <= 0) return "mlstm_hip_recurrent_sequence: non-positive dimension";
   if ((long long)B * NH > 65535) return "mlstm_hip_recurrent_sequence: B*NH exceeds 65535";
   if (DHQK > 1024) return "mlstm_hip_recurrent_sequence: DHQK above 1024 does not fit the register-resident state slice";
-#define MLSTM_SEQ_ARGS q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, T, DHQK, DHHV, eps, dtype_qkv, dtype_gates, stream
+#define MLSTM_SEQ_ARGS q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, T, DHQK, DHHV, eps, dtype_qkv, dtype_gates, dtype_state, stream
   // rows per lane x columns per lane: at most 128 state registers per lane
   const bool vec = DHHV % 4 == 0, bf = dtype_qkv != 0;
 #define MLSTM_SEQ_PICK(RPT_, CPT_, VEC_) \

@@ -11,6 +11,14 @@ from ... import _lib
 from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu
 
 
+def _check_state_dtype(dtype_state: torch.dtype) -> torch.dtype:
+    """The states are kept in float32 or bfloat16 (the arithmetic is float32 either way); the reference's third choice,
+    float16 (mlstm_kernels/torch/backend_module.py:80-82 inference_state_dtype), has no kernel here."""
+    if dtype_state not in (torch.float32, torch.bfloat16):
+        raise NotImplementedError(f"the HIP step kernels keep the recurrent state in float32 or bfloat16, not {dtype_state}")
+    return dtype_state
+
+
 def mlstm_recurrent_step__hip_fw(
     matC_old: torch.Tensor,  # (B, NH, DHQK, DHHV)
     vecN_old: torch.Tensor,  # (B, NH, DHQK)
@@ -40,16 +48,15 @@ def mlstm_recurrent_step__hip_fw(
     assert scaF.shape == (B, NH, 1), f"scaF has wrong shape, got {scaF.shape}"
     if qk_scale is not None and abs(qk_scale - DHQK ** -0.5) > 1e-12:
         raise NotImplementedError("the HIP step kernel uses qk_scale = DHQK**-0.5")
-    if dtype_state != torch.float32:
-        raise NotImplementedError("the HIP step kernel keeps the recurrent state in float32")
+    dtype_state = _check_state_dtype(dtype_state)
     dev = require_gpu(vecQ, vecK, vecV, scaI, scaF, matC_old, vecN_old, scaM_old)
     q, k, v = vecQ.contiguous(), vecK.contiguous(), vecV.to(vecQ.dtype).contiguous()
     if k.dtype != q.dtype:
         k = k.to(q.dtype)
     i, f = scaI.contiguous(), scaF.to(scaI.dtype).contiguous()
-    c_old = matC_old.to(torch.float32).contiguous()
-    n_old = vecN_old.to(torch.float32).contiguous()
-    m_old = scaM_old.to(torch.float32).contiguous()
+    c_old = matC_old.to(dtype_state).contiguous()
+    n_old = vecN_old.to(dtype_state).contiguous()
+    m_old = scaM_old.to(dtype_state).contiguous()
     if matC_new is None:
         assert vecN_new is None and scaM_new is None, "Initial states must be provided together."
         matC_new = torch.empty_like(c_old)
@@ -58,13 +65,13 @@ def mlstm_recurrent_step__hip_fw(
     else:
         assert vecN_new is not None and scaM_new is not None, "Initial states must be provided together."
         for t in (matC_new, vecN_new, scaM_new):
-            assert t.dtype == torch.float32 and t.is_contiguous(), "state outputs must be contiguous float32"
+            assert t.dtype == dtype_state and t.is_contiguous(), f"state outputs must be contiguous {dtype_state}"
     h = torch.empty_like(v)
     lib = _lib.get_lib()
     rc = lib.mlstm_hip_step(
         ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c_old), ptr(n_old), ptr(m_old),
         ptr(h), ptr(matC_new), ptr(vecN_new), ptr(scaM_new),
-        B, NH, DHQK, DHHV, float(eps), dtype_code(q), dtype_code(i), current_stream_ptr(dev),
+        B, NH, DHQK, DHHV, float(eps), dtype_code(q), dtype_code(i), dtype_code(c_old), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_step")
     return h, (matC_new, vecN_new, scaM_new)
@@ -113,20 +120,19 @@ def mlstm_recurrent_sequence__hip(
     assert k.shape == q.shape, "q and k must have the same shape"
     assert v.shape[:3] == (B, NH, S), f"v has wrong shape, got {v.shape}"
     assert i.shape == (B, NH, S) and f.shape == (B, NH, S), "i and f must have shape (B, NH, S)"
-    if dtype_state != torch.float32:
-        raise NotImplementedError("the HIP step kernels keep the recurrent state in float32")
+    dtype_state = _check_state_dtype(dtype_state)
     dev = require_gpu(q, k, v, i, f)
     if c_initial is not None:
         assert n_initial is not None and m_initial is not None, "Initial states must be provided together."
-        c = c_initial.to(torch.float32).contiguous()
-        n = n_initial.to(torch.float32).contiguous()
-        m = m_initial.to(torch.float32).contiguous().reshape(B, NH, 1)
+        c = c_initial.to(dtype_state).contiguous()
+        n = n_initial.to(dtype_state).contiguous()
+        m = m_initial.to(dtype_state).contiguous().reshape(B, NH, 1)
         assert c.shape == (B, NH, DHQK, DHHV), f"c_initial has wrong shape, got {c.shape}"
         assert n.shape == (B, NH, DHQK), f"n_initial has wrong shape, got {n.shape}"
     else:
-        c = torch.zeros(B, NH, DHQK, DHHV, dtype=torch.float32, device=dev)
-        n = torch.zeros(B, NH, DHQK, dtype=torch.float32, device=dev)
-        m = torch.zeros(B, NH, 1, dtype=torch.float32, device=dev)
+        c = torch.zeros(B, NH, DHQK, DHHV, dtype=dtype_state, device=dev)
+        n = torch.zeros(B, NH, DHQK, dtype=dtype_state, device=dev)
+        m = torch.zeros(B, NH, 1, dtype=dtype_state, device=dev)
     if S == 0:
         H = torch.empty(B, NH, 0, DHHV, dtype=q.dtype, device=dev)
         return (H, (c.clone(), n.clone(), m.clone())) if return_last_states else H
@@ -138,7 +144,7 @@ def mlstm_recurrent_sequence__hip(
     rc = lib.mlstm_hip_recurrent_sequence(
         ptr(qc), ptr(kc), ptr(vc), ptr(ic), ptr(fc), ptr(c), ptr(n), ptr(m),
         ptr(H), ptr(c_out), ptr(n_out), ptr(m_out),
-        B, NH, S, DHQK, DHHV, float(eps), dtype_code(qc), dtype_code(ic), current_stream_ptr(dev),
+        B, NH, S, DHQK, DHHV, float(eps), dtype_code(qc), dtype_code(ic), dtype_code(c), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_recurrent_sequence")
     if return_last_states:

@@ -110,7 +110,7 @@ def test_library_exports_every_declared_symbol():
     assert full - half == 2 * 16 * 256 * 512 * 2
     assert lib.mlstm_hip_chunkwise_bw_workspace_bytes(1, 2, 256, 64, 128, 0) > 0
     rc = lib.mlstm_hip_step(None, None, None, None, None, None, None, None, None, None, None, None,
-                            1, 1, 64, 64, 1e-6, 1, 0, None)
+                            1, 1, 64, 64, 1e-6, 1, 0, 0, None)
     assert rc != 0 and b"null pointer" in lib.mlstm_hip_last_error()
 
 

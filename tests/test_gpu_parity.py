@@ -189,20 +189,72 @@ def test_recurrent_sequence_parity(B, NH, T, DQK, DHV, dtype, init):
     assert_state_close(n2, d64(n), 1e-6, "n vs step loop")
 
 
+@pytest.mark.parametrize("B,NH,DQK,DHV", [(2, 2, 64, 128), (3, 4, 256, 512), (1, 2, 96, 104), (88, 8, 256, 512),
+                                          (162, 8, 256, 512)])
+def test_step_parity_bf16_state(B, NH, DQK, DHV):
+    """States kept in bfloat16 (the reference's dtype_state, triton_step.py:33,67-69): the kernel reads bf16 C, n, m,
+    computes in fp32 and rounds the new states once.  Oracle: the fp64 step on the same bf16-rounded inputs; the new
+    states must lie within one unit in the last place of bfloat16 (at most 2^-7 relative) of the fp64 values, h comes
+    from the unrounded state.  (162, 8, 256, 512) is a 340 MB bf16 state: the streaming variant.)"""
+    *_, step, _ = _ops()
+    g = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(B, NH, d, generator=g).bfloat16() for d in (DQK, DQK, DHV))
+    i, f = torch.randn(B, NH, 1, generator=g), 3 + torch.randn(B, NH, 1, generator=g)
+    c = torch.randn(B, NH, DQK, DHV, generator=g).bfloat16()
+    n, m = torch.randn(B, NH, DQK, generator=g).bfloat16(), torch.randn(B, NH, 1, generator=g).bfloat16()
+    h_r, (c_r, n_r, m_r) = O.recurrent_step(*(d64(t) for t in (q, k, v, i, f, c, n, m)))
+    h, (c2, n2, m2) = step(*(t.to(DEV) for t in (q, k, v, i, f, c, n, m)), dtype_state=torch.bfloat16)
+    assert c2.dtype == n2.dtype == m2.dtype == torch.bfloat16 and h.dtype == torch.bfloat16
+    assert rel_to_scale(h, h_r) <= 5e-3
+    for name, x, ref in (("C", c2, c_r), ("n", n2, n_r), ("m", m2, m_r)):
+        err = (d64(x) - ref).abs()
+        # (+ fp32 rounding of the two products on elements where they nearly cancel)
+        assert bool((err <= 2.0 ** -7 * ref.abs() + 1e-6 * float(ref.abs().max())).all()), (
+            f"{name}: more than one bf16 ulp off (max {float(err.max()):.3e})")
+    # in place
+    c_dev = c.to(DEV).clone()
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw
+    n_new, m_new = torch.empty_like(n2), torch.empty_like(m2)
+    h3, (c3, _, _) = mlstm_recurrent_step__hip_fw(c_dev, n.to(DEV), m.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), i.to(DEV),
+                                                  f.to(DEV), matC_new=c_dev, vecN_new=n_new, scaM_new=m_new,
+                                                  dtype_state=torch.bfloat16)
+    assert c3.data_ptr() == c_dev.data_ptr() and torch.equal(c3, c2) and torch.equal(h3, h)
+
+
+@pytest.mark.parametrize("B,NH,T,DQK,DHV", [(2, 2, 9, 64, 128), (3, 4, 33, 256, 512), (1, 2, 5, 96, 100), (1, 1, 4, 384, 64)])
+def test_recurrent_sequence_bf16_state(B, NH, T, DQK, DHV):
+    """bf16 states in and out of the multi-token kernel: fp32 between the tokens, rounded once at the end."""
+    *_, seq = _ops()
+    g = torch.Generator().manual_seed(13)
+    q, k, v = (torch.randn(B, NH, T, d, generator=g).bfloat16() for d in (DQK, DQK, DHV))
+    i, f = torch.randn(B, NH, T, generator=g), 3 + torch.randn(B, NH, T, generator=g)
+    c0 = torch.randn(B, NH, DQK, DHV, generator=g).bfloat16()
+    n0, m0 = torch.randn(B, NH, DQK, generator=g).bfloat16(), torch.randn(B, NH, 1, generator=g).bfloat16()
+    H_r, (c_r, n_r, m_r) = O.recurrent_sequence(*(d64(t) for t in (q, k, v, i, f)), c_initial=d64(c0), n_initial=d64(n0),
+                                                m_initial=d64(m0))
+    H, (c2, n2, m2) = seq(*(t.to(DEV) for t in (q, k, v, i, f)), c_initial=c0.to(DEV), n_initial=n0.to(DEV),
+                          m_initial=m0.to(DEV), return_last_states=True, dtype_state=torch.bfloat16)
+    assert c2.dtype == n2.dtype == m2.dtype == torch.bfloat16
+    assert rel_to_scale(H, H_r) <= 5e-3
+    for name, x, ref in (("C", c2, c_r), ("n", n2, n_r), ("m", m2, m_r)):
+        err = (d64(x) - ref).abs()
+        assert bool((err <= 2.0 ** -7 * ref.abs() + 1e-5 * float(ref.abs().max())).all()), f"{name}: max error {float(err.max()):.3e}"
+
+
 def test_recurrent_sequence_rejects_bad_arguments():
     from mlstm_kernels_amd import _lib
     lib = _lib.get_lib()
     z = torch.zeros(64, device=DEV)
     p = z.data_ptr()
     # aliasing n / m, unsupported dtype code, DHQK beyond the register-resident slice, no tokens
-    assert lib.mlstm_hip_recurrent_sequence(p, p, p, p, p, p, p, p, p, p, p, p, 1, 1, 1, 4, 4, 1e-6, 0, 0, None) != 0
+    assert lib.mlstm_hip_recurrent_sequence(p, p, p, p, p, p, p, p, p, p, p, p, 1, 1, 1, 4, 4, 1e-6, 0, 0, 0, None) != 0
     assert b"alias" in lib.mlstm_hip_last_error()
     n2, m2 = torch.zeros(64, device=DEV), torch.zeros(64, device=DEV)
     args = lambda *dims_dt: (p, p, p, p, p, p, p, p, p, p, n2.data_ptr(), m2.data_ptr(), *dims_dt, None)
-    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 1, 4, 4, 1e-6, 7, 0)) != 0
-    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 1, 2048, 4, 1e-6, 0, 0)) != 0
+    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 1, 4, 4, 1e-6, 7, 0, 0)) != 0
+    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 1, 2048, 4, 1e-6, 0, 0, 0)) != 0
     assert b"1024" in lib.mlstm_hip_last_error()
-    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 0, 4, 4, 1e-6, 0, 0)) != 0
+    assert lib.mlstm_hip_recurrent_sequence(*args(1, 1, 0, 4, 4, 1e-6, 0, 0, 0)) != 0
 
 
 @pytest.mark.parametrize("B", [16, 64, 256])
@@ -524,6 +576,13 @@ def test_backend_module_hip_train_and_inference():
     h1_r, (c1_r, _, _) = O.recurrent_step(d64(q1[:, :, 0]), d64(k1[:, :, 0]), d64(v1[:, :, 0]), d64(i1), d64(f1), c_r, n_r, m_r)
     assert h1.shape == (2, 2, 1, 128) and allclose_frac(h1[:, :, 0], h1_r, 2e-2, 2e-2) == 0.0
     assert_state_close(C1, c1_r, 1e-3, "C after step")
+    # the same with the states of the generation phase kept in bfloat16 (inference_state_dtype of the reference,
+    # mlstm_kernels/torch/backend_module.py:80-82): the state tolerance is one bf16 unit, h is unaffected
+    backend_bf = mLSTMBackend(mLSTMBackendConfig(chunk_size=128, mode="inference", inference_state_dtype="bfloat16")).to(DEV)
+    h1b, (C1b, n1b, m1b) = backend_bf(*(t.to(DEV) for t in (q1, k1, v1, i1, f1)), C, n, m)
+    assert C1b.dtype == torch.bfloat16 and n1b.dtype == torch.bfloat16
+    assert allclose_frac(h1b[:, :, 0], h1_r, 3e-2, 3e-2) == 0.0
+    assert_state_close(C1b, c1_r, 1e-2, "bf16 C after step")
     # train mode, padded train mode, sigmoid gate through the module
     train = mLSTMBackend(mLSTMBackendConfig(chunk_size=128, mode="train"))
     qq, kk, vv, ii, ff = (t[:, :, :256].contiguous().to(DEV) for t in (q, k, v, i, f))
