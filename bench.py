@@ -17,6 +17,8 @@ Objects on the JSON line besides the contract's keys:
   roofline      -- the chunkwise kernel with the largest share of the step against the bf16 MFMA peak: algorithmic
                    flops of one launch / its average duration; `traffic` = measured HBM bytes per launch, parsed from
                    the rocprofv3 counter summary under profiles/ (null when that file has no row for the kernel).
+  peak_memory_gb -- peak device memory of one forward+backward pass (inputs, outputs, gradients, workspaces; without
+                   the benchmark's own flush buffer); the reference's benchmark reports 9.0-9.9 GB for this workload.
   roofline_hbm  -- the same kernel against the HBM peak (algorithmic bytes per launch).
   kernels       -- average duration, algorithmic TFLOP/s and GB/s of every kernel of the step.
   decode_step   -- fused decode step at B=256 after a chunkwise prefill of 2048 positions: ms per step, algorithmic
@@ -215,6 +217,16 @@ def main():
             prepare()
             step()
         torch.cuda.synchronize()
+        # peak device memory of one pass beyond what is allocated before it (inputs, upstream gradient, flush buffer):
+        # the output, the gradients and the library's workspaces -- the quantity the reference's benchmark reports
+        prepare()
+        torch.cuda.synchronize()
+        base_mem = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()
+        step()
+        torch.cuda.synchronize()
+        peak_extra = torch.cuda.max_memory_allocated() - base_mem
+        peak_total = torch.cuda.max_memory_allocated() - flush.numel()
         events = []
         t0 = time.perf_counter()
         for _ in range(steps):
@@ -237,7 +249,8 @@ def main():
         torch.cuda.synchronize()
         _lib.profile_enable(False)
         kern = {name: (ms / max(cnt, 1), cnt) for name, (ms, cnt) in _lib.profile_read().items()}
-        return {"median_ms": median, "mean_ms": mean, "min_ms": times[0], "wall_ms_incl_flush": wall / steps * 1e3, "kernels": kern}
+        return {"median_ms": median, "mean_ms": mean, "min_ms": times[0], "wall_ms_incl_flush": wall / steps * 1e3, "kernels": kern,
+                "peak_memory_gb": round(peak_total / 1e9, 3), "peak_memory_beyond_inputs_gb": round(peak_extra / 1e9, 3)}
 
     def kernel_table(kern, token_heads, alg_bytes=None):
         table = {}
@@ -283,6 +296,7 @@ def main():
             fl = (FLOPS_FW + (FLOPS_BW if cfg.get("backward", True) else 0)) * TOKEN_HEADS
             extra[tag] = {"ms_per_step": round(r["median_ms"], 4), "steps": n_extra,
                           "value": round(fl / (r["median_ms"] * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                          "peak_memory_gb": r["peak_memory_gb"],
                           "kernels": kernel_table(r["kernels"], TOKEN_HEADS)}
             torch.cuda.empty_cache()
     del flush
@@ -416,6 +430,7 @@ def main():
         "timing": {"protocol": "median of per-step HIP-event times, 512 MB cache flush and gradient reset before every step",
                    "mean_ms": round(head["mean_ms"], 4), "min_ms": round(head["min_ms"], 4),
                    "wall_ms_per_step_incl_flush": round(head["wall_ms_incl_flush"], 4)},
+        "peak_memory_gb": head["peak_memory_gb"], "peak_memory_beyond_inputs_gb": head["peak_memory_beyond_inputs_gb"],
         "roofline": roofline, "roofline_hbm": roofline_hbm, "kernels": kernels, "decode_step": decode, "extra": extra,
     }
     if not args.no_cpu_baseline:
