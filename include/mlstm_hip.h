@@ -10,7 +10,7 @@
  *     C (B,NH,DHQK,DHHV) fp32; n (B,NH,DHQK) fp32; m (B,NH) fp32.
  *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it.
  *   - Return value 0 = success; anything else = failure, message via mlstm_hip_last_error().
- *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1.  gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp),
+ *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1 (and MLSTM_F16 = 2 for the recurrent states only).  gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp),
  *     MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
  *   - Supported shapes: DHQK % 64 == 0 (at most 896), DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
  *
@@ -28,6 +28,7 @@ extern "C" {
 
 #define MLSTM_F32 0
 #define MLSTM_BF16 1
+#define MLSTM_F16 2 /* recurrent states only (dtype_state) */
 #define MLSTM_GATE_EXP 0
 #define MLSTM_GATE_SIG 1
 
@@ -92,9 +93,9 @@ const char* mlstm_hip_last_error(void);
  * Replaces: mlstm_kernels/torch/recurrent/triton_step.py:15-127 (mlstm_recurrent_step__triton_fw) and the
  * Triton kernel mlstm_kernels/triton/recurrent/fw_step_fused.py:19-195.
  *   q,k (B,NH,DHQK), v (B,NH,DHHV) in dtype_qkv; i,f (B,NH) in dtype_gates; h (B,NH,DHHV) in dtype_qkv.
- *   States C (B,NH,DHQK,DHHV), n (B,NH,DHQK), m (B,NH) in and out in dtype_state (MLSTM_F32 or MLSTM_BF16: the
+ *   States C (B,NH,DHQK,DHHV), n (B,NH,DHQK), m (B,NH) in and out in dtype_state (MLSTM_F32, MLSTM_BF16 or MLSTM_F16: the
  *   reference's dtype_state, triton_step.py:33,67-69); the arithmetic is fp32 either way, h is formed from the
- *   unrounded new state.  DHHV % 4 == 0 (fp32 state) or % 8 == 0 (bf16 state).
+ *   unrounded new state.  DHHV % 4 == 0 (fp32 state) or % 8 == 0 (16-bit state).
  *   c_out may alias c_in (in-place update of the state matrix); n_out/m_out must be distinct from n_in/m_in
  *   (every workgroup of a head reads the old n and m while one of them writes the new values).
  */

@@ -140,7 +140,7 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
   if (n_out == n_in || m_out == m_in)
     return fail("mlstm_hip_step: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
   if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) ||
-      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16))
+      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16 && dtype_state != MLSTM_F16))
     return fail("mlstm_hip_step: unsupported dtype code");
   {
     ProfileScope ps("step", (hipStream_t)stream);
@@ -160,7 +160,7 @@ int mlstm_hip_recurrent_sequence(const void* q, const void* k, const void* v, co
   if (n_out == n_in || m_out == m_in)
     return fail("mlstm_hip_recurrent_sequence: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
   if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) ||
-      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16))
+      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16 && dtype_state != MLSTM_F16))
     return fail("mlstm_hip_recurrent_sequence: unsupported dtype code");
   {
     ProfileScope ps("step_seq", (hipStream_t)stream);

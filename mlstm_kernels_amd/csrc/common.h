@@ -93,6 +93,35 @@ __device__ __forceinline__ float load_scalar(const void* p, size_t idx, int dtyp
   return dtype == 0 ? ((const float*)p)[idx] : bf16_bits_to_f32(((const uint16_t*)p)[idx]);
 }
 
+// Recurrent states may be kept in float32 (0), bfloat16 (1) or float16 (2); the arithmetic is float32.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float load_state_scalar(const void* p, size_t idx, int sdt) {
+  if (sdt == 0) return ((const float*)p)[idx];
+  if (sdt == 1) return bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+  return (float)((const _Float16*)p)[idx];
+}
+__device__ __forceinline__ void store_state_scalar(void* p, size_t idx, int sdt, float x) {
+  if (sdt == 0) ((float*)p)[idx] = x;
+  else if (sdt == 1) ((uint16_t*)p)[idx] = f32_to_bf16_bits(x);
+  else ((_Float16*)p)[idx] = (_Float16)x;
+}
+// two 16-bit state values packed in one 32-bit word (sdt = 1 or 2)
+__device__ __forceinline__ void unpack_state2(uint32_t w, int sdt, float& lo, float& hi) {
+  if (sdt == 1) {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+  } else {
+    const f16x2 hv = __builtin_bit_cast(f16x2, w);
+    lo = (float)hv[0];
+    hi = (float)hv[1];
+  }
+}
+__device__ __forceinline__ uint32_t pack_state2(float lo, float hi, int sdt) {
+  if (sdt == 1) return pack_bf16x2(lo, hi);
+  const f16x2 hv = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, hv);
+}
+
 // XCD-aware workgroup renumbering.  The hardware deals consecutive linear workgroup ids round-robin to the 8
 // XCDs (each with its own L2).  Mapping linear id -> (id % 8) * (total / 8) + id / 8 gives every XCD a
 // contiguous range of virtual ids, so neighbouring tiles (which share operands) share an L2.

@@ -17,24 +17,22 @@
 
 namespace mlstm {
 
-// One 16-byte piece of a state row: four fp32 columns, or eight bf16 columns when the state is kept in bfloat16
+// One 16-byte piece of a state row: four fp32 columns, or eight columns when the state is kept in bfloat16 or float16
 // (the reference's dtype_state / inference_state_dtype, mlstm_kernels/torch/recurrent/triton_step.py:33,67-69).
-template <bool SBF>
+// SBF = state dtype code: 0 float32, 1 bfloat16, 2 float16.
+template <int SBF>
 struct StatePiece {
   static constexpr int N = SBF ? 8 : 4;
   float x[N];
 };
-template <bool SBF, bool NT>
+template <int SBF, bool NT>
 __device__ __forceinline__ StatePiece<SBF> load_piece(const void* base, size_t elem) {
   StatePiece<SBF> p;
-  if constexpr (SBF) {
+  if constexpr (SBF != 0) {
     const u32x4* src = (const u32x4*)((const uint16_t*)base + elem);
     const u32x4 raw = NT ? __builtin_nontemporal_load(src) : *src;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      p.x[2 * e] = __uint_as_float(raw[e] << 16);
-      p.x[2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u);
-    }
+    for (int e = 0; e < 4; ++e) unpack_state2(raw[e], SBF, p.x[2 * e], p.x[2 * e + 1]);
   } else {
     const f32x4* src = (const f32x4*)((const float*)base + elem);
     const f32x4 raw = NT ? __builtin_nontemporal_load(src) : *src;
@@ -43,11 +41,11 @@ __device__ __forceinline__ StatePiece<SBF> load_piece(const void* base, size_t e
   }
   return p;
 }
-template <bool SBF, bool NT>
+template <int SBF, bool NT>
 __device__ __forceinline__ void store_piece(void* base, size_t elem, const StatePiece<SBF>& p) {
-  if constexpr (SBF) {
-    const u32x4 raw = {pack_bf16x2(p.x[0], p.x[1]), pack_bf16x2(p.x[2], p.x[3]), pack_bf16x2(p.x[4], p.x[5]),
-                       pack_bf16x2(p.x[6], p.x[7])};
+  if constexpr (SBF != 0) {
+    const u32x4 raw = {pack_state2(p.x[0], p.x[1], SBF), pack_state2(p.x[2], p.x[3], SBF), pack_state2(p.x[4], p.x[5], SBF),
+                       pack_state2(p.x[6], p.x[7], SBF)};
     u32x4* dst = (u32x4*)((uint16_t*)base + elem);
     if (NT) __builtin_nontemporal_store(raw, dst);
     else *dst = raw;
@@ -59,7 +57,7 @@ __device__ __forceinline__ void store_piece(void* base, size_t elem, const State
   }
 }
 
-template <int COLS, int TY, int UNROLL, bool NONTEMPORAL, bool SBF>
+template <int COLS, int TY, int UNROLL, bool NONTEMPORAL, int SBF>
 __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
     const void* __restrict__ ig, const void* __restrict__ fg,
@@ -69,7 +67,7 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
   constexpr int VPL = StatePiece<SBF>::N;   // state columns per lane
   constexpr int TX = COLS / VPL;
   constexpr int NTH = TX * TY;
-  constexpr int dtype_state = SBF ? 1 : 0;
+  constexpr int dtype_state = SBF;
   extern __shared__ float smem[];
   float* qs = smem;                 // [DHQK] q / sqrt(d)
   float* ik = smem + DHQK;          // [DHQK] i' * k
@@ -101,7 +99,7 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
 
   const float fpre = load_scalar(fg, bh, dtype_gates);
   const float ipre = load_scalar(ig, bh, dtype_gates);
-  const float m_old = load_scalar(m_in, bh, dtype_state);
+  const float m_old = load_state_scalar(m_in, bh, dtype_state);
   const float lf = log_sigmoid(fpre);
   const float m_new = fmaxf(lf + m_old, ipre);
   const float fa = expf(lf + m_old - m_new);
@@ -114,14 +112,11 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
     const size_t o = (size_t)bh * DHQK + d;
     const float qd = load_scalar(q, o, dtype_qkv) * scale;
     const float kd = load_scalar(k, o, dtype_qkv);
-    const float nd = fa * load_scalar(n_in, o, dtype_state) + ia * kd;
+    const float nd = fa * load_state_scalar(n_in, o, dtype_state) + ia * kd;
     qs[d] = qd;
     ik[d] = ia * kd;
     qn_part += qd * nd;
-    if (blockIdx.x == 0) {
-      if (SBF) ((uint16_t*)n_out)[o] = f32_to_bf16_bits(nd);
-      else ((float*)n_out)[o] = nd;
-    }
+    if (blockIdx.x == 0) store_state_scalar(n_out, o, dtype_state, nd);
   }
   qn_part = wave_sum(qn_part);
   __shared__ float wsum[(NTH + kWave - 1) / kWave];
@@ -131,10 +126,7 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
 #pragma unroll
   for (int w = 0; w < (NTH + kWave - 1) / kWave; ++w) qn += wsum[w];
   const float inv_den = 1.f / (fmaxf(fabsf(qn), expf(-m_new)) + eps);
-  if (blockIdx.x == 0 && tid == 0) {
-    if (SBF) ((uint16_t*)m_out)[bh] = f32_to_bf16_bits(m_new);
-    else ((float*)m_out)[bh] = m_new;
-  }
+  if (blockIdx.x == 0 && tid == 0) store_state_scalar(m_out, bh, dtype_state, m_new);
 
   float vv[VPL];
 #pragma unroll
@@ -214,7 +206,7 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
   }
 }
 
-template <int COLS, int TY, int UNROLL, bool NONTEMPORAL, bool SBF>
+template <int COLS, int TY, int UNROLL, bool NONTEMPORAL, int SBF>
 static const char* launch_step_t(const void* q, const void* k, const void* v, const void* i, const void* f,
                                  const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
                                  void* n_out, void* m_out, int B, int NH, int DHQK, int DHHV, float eps,
@@ -235,23 +227,27 @@ const char* launch_step(const void* q, const void* k, const void* v, const void*
   if (B <= 0 || NH <= 0 || DHQK <= 0 || DHHV <= 0) return "mlstm_hip_step: non-positive dimension";
   const bool sbf = dtype_state != 0;
   if (DHHV % (sbf ? 8 : 4) != 0)
-    return sbf ? "mlstm_hip_step: DHHV must be a multiple of 8 for a bfloat16 state" : "mlstm_hip_step: DHHV must be a multiple of 4";
+    return sbf ? "mlstm_hip_step: DHHV must be a multiple of 8 for a 16-bit state" : "mlstm_hip_step: DHHV must be a multiple of 4";
   if ((long long)B * NH > 65535) return "mlstm_hip_step: B*NH exceeds 65535";
   // Tile shapes from a sweep on MI355X (B = 16/64/256, NH = 8, 256 x 512 fp32 state).  A state larger than the 256 MB
   // memory-side cache streams past the caches with non-temporal accesses: 256-column slices, 8 row groups, 16 rows
   // in flight per lane.  A smaller one is best left cacheable (it is re-read by the next step) and has few
   // workgroups per CU: 128-column slices with 16 row groups, the first 16 rows per lane requested before the
   // prologue.  The crossover was measured between a 268 MB state (cacheable 79 us, streaming 90 us) and a 403 MB
-  // state (156 us against 133 us).  A bfloat16 state uses the same shapes with lanes of eight columns (half as many
+  // state (156 us against 133 us).  A bfloat16 or float16 state uses the same shapes with lanes of eight columns (half as many
   // lanes per row segment), so every lane still moves 16 bytes per access.
   const size_t state_bytes = (size_t)B * NH * DHQK * DHHV * (sbf ? 2 : 4);
   const bool stream_past_cache = state_bytes > ((size_t)320 << 20);
 #define MLSTM_STEP_ARGS q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, DHQK, DHHV, eps, dtype_qkv, dtype_gates, stream
-#define MLSTM_STEP_PICK(COLS_, TY_, UN_, NT_) \
-  return sbf ? launch_step_t<COLS_, TY_, UN_, NT_, true>(MLSTM_STEP_ARGS) : launch_step_t<COLS_, TY_, UN_, NT_, false>(MLSTM_STEP_ARGS)
-  if (DHHV % 256 == 0 && stream_past_cache) MLSTM_STEP_PICK(256, 8, 16, true);
-  if (stream_past_cache) MLSTM_STEP_PICK(128, 8, 8, true);
-  MLSTM_STEP_PICK(128, 16, 16, false);
+#define MLSTM_STEP_PICK(COLS_, TY_, UN_, NT_)                                                          \
+  {                                                                                                     \
+    if (dtype_state == 1) return launch_step_t<COLS_, TY_, UN_, NT_, 1>(MLSTM_STEP_ARGS);               \
+    if (dtype_state == 2) return launch_step_t<COLS_, TY_, UN_, NT_, 2>(MLSTM_STEP_ARGS);               \
+    return launch_step_t<COLS_, TY_, UN_, NT_, 0>(MLSTM_STEP_ARGS);                                      \
+  }
+  if (DHHV % 256 == 0 && stream_past_cache) MLSTM_STEP_PICK(256, 8, 16, true)
+  if (stream_past_cache) MLSTM_STEP_PICK(128, 8, 8, true)
+  MLSTM_STEP_PICK(128, 16, 16, false)
 #undef MLSTM_STEP_PICK
 #undef MLSTM_STEP_ARGS
 }

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(64)
   // (loads are unconditional from clamped addresses, the result is selected afterwards: no branches around them)
   float C[RPT][CPT];
   const bool col_in = col < DHHV;
-  const bool sbf = dtype_state != 0;  // states in and out in bfloat16 (fp32 in registers between the tokens)
+  const bool sbf = dtype_state != 0;  // states in and out in bfloat16 or float16 (fp32 in registers between the tokens)
 #pragma unroll
   for (int u = 0; u < RPT; ++u) {
     const int r = g * RPT + u;
@@ -87,10 +87,8 @@ __global__ __launch_bounds__(64)
       float x[4];
       if (sbf) {
         const uint2 raw = *(const uint2*)((const uint16_t*)c_in + row + (col_in ? col : 0));
-        x[0] = __uint_as_float(raw.x << 16);
-        x[1] = __uint_as_float(raw.x & 0xffff0000u);
-        x[2] = __uint_as_float(raw.y << 16);
-        x[3] = __uint_as_float(raw.y & 0xffff0000u);
+        unpack_state2(raw.x, dtype_state, x[0], x[1]);
+        unpack_state2(raw.y, dtype_state, x[2], x[3]);
       } else {
         const f32x4 raw = *(const f32x4*)((const float*)c_in + row + (col_in ? col : 0));
 #pragma unroll
@@ -101,7 +99,7 @@ __global__ __launch_bounds__(64)
     } else {
 #pragma unroll
       for (int e = 0; e < CPT; ++e) {
-        const float x = load_scalar(c_in, row + min(col + e, DHHV - 1), dtype_state);
+        const float x = load_state_scalar(c_in, row + min(col + e, DHHV - 1), dtype_state);
         C[u][e] = (r < DHQK && col + e < DHHV) ? x : 0.f;
       }
     }
@@ -110,13 +108,13 @@ __global__ __launch_bounds__(64)
 #pragma unroll
   for (int j = 0; j < NDJ; ++j) {
     const int d = lane + j * kWave;
-    nreg[j] = d < DHQK ? load_scalar(n_in, (size_t)bh * DHQK + d, dtype_state) : 0.f;
+    nreg[j] = d < DHQK ? load_state_scalar(n_in, (size_t)bh * DHQK + d, dtype_state) : 0.f;
   }
   for (int x = lane; x < 2 * NG * RS; x += kWave) {
     (&qs[0][0])[x] = 0.f;
     (&ik[0][0])[x] = 0.f;
   }
-  float m = load_scalar(m_in, bh, dtype_state);
+  float m = load_state_scalar(m_in, bh, dtype_state);
 
   // ---- token inputs, PF tokens ahead, in a ring that is shifted by one slot per token.  Tokens past the end
   // re-request the last one (nobody uses them): an unconditional load keeps the ring in registers.
@@ -318,7 +316,7 @@ __global__ __launch_bounds__(64)
         if (col_in) {
           if (sbf) {
             *(uint2*)((uint16_t*)c_out + row + col) =
-                make_uint2(pack_bf16x2(C[u][0], C[u][1 % CPT]), pack_bf16x2(C[u][2 % CPT], C[u][3 % CPT]));
+                make_uint2(pack_state2(C[u][0], C[u][1 % CPT], dtype_state), pack_state2(C[u][2 % CPT], C[u][3 % CPT], dtype_state));
           } else {
             const f32x4 y = {C[u][0], C[u][1 % CPT], C[u][2 % CPT], C[u][3 % CPT]};
             *(f32x4*)((float*)c_out + row + col) = y;
@@ -327,10 +325,7 @@ __global__ __launch_bounds__(64)
       } else {
 #pragma unroll
         for (int e = 0; e < CPT; ++e)
-          if (col + e < DHHV) {
-            if (sbf) ((uint16_t*)c_out)[row + col + e] = f32_to_bf16_bits(C[u][e]);
-            else ((float*)c_out)[row + col + e] = C[u][e];
-          }
+          if (col + e < DHHV) store_state_scalar(c_out, row + col + e, dtype_state, C[u][e]);
       }
     }
   }
@@ -338,15 +333,9 @@ __global__ __launch_bounds__(64)
 #pragma unroll
     for (int j = 0; j < NDJ; ++j) {
       const int d = lane + j * kWave;
-      if (d < DHQK) {
-        if (sbf) ((uint16_t*)n_out)[(size_t)bh * DHQK + d] = f32_to_bf16_bits(nreg[j]);
-        else ((float*)n_out)[(size_t)bh * DHQK + d] = nreg[j];
-      }
+      if (d < DHQK) store_state_scalar(n_out, (size_t)bh * DHQK + d, dtype_state, nreg[j]);
     }
-    if (lane == 0) {
-      if (sbf) ((uint16_t*)m_out)[bh] = f32_to_bf16_bits(m);
-      else ((float*)m_out)[bh] = m;
-    }
+    if (lane == 0) store_state_scalar(m_out, bh, dtype_state, m);
   }
 }
 

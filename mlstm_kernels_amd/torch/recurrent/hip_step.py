@@ -8,14 +8,14 @@ from __future__ import annotations
 import torch
 
 from ... import _lib
-from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu
+from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu, state_dtype_code
 
 
 def _check_state_dtype(dtype_state: torch.dtype) -> torch.dtype:
-    """The states are kept in float32 or bfloat16 (the arithmetic is float32 either way); the reference's third choice,
-    float16 (mlstm_kernels/torch/backend_module.py:80-82 inference_state_dtype), has no kernel here."""
-    if dtype_state not in (torch.float32, torch.bfloat16):
-        raise NotImplementedError(f"the HIP step kernels keep the recurrent state in float32 or bfloat16, not {dtype_state}")
+    """The states are kept in float32, bfloat16 or float16 -- the choices of the reference's inference_state_dtype
+    (mlstm_kernels/torch/backend_module.py:38,75); the arithmetic is float32 either way."""
+    if dtype_state not in (torch.float32, torch.bfloat16, torch.float16):
+        raise NotImplementedError(f"the HIP step kernels keep the recurrent state in float32, bfloat16 or float16, not {dtype_state}")
     return dtype_state
 
 
@@ -71,7 +71,7 @@ def mlstm_recurrent_step__hip_fw(
     rc = lib.mlstm_hip_step(
         ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c_old), ptr(n_old), ptr(m_old),
         ptr(h), ptr(matC_new), ptr(vecN_new), ptr(scaM_new),
-        B, NH, DHQK, DHHV, float(eps), dtype_code(q), dtype_code(i), dtype_code(c_old), current_stream_ptr(dev),
+        B, NH, DHQK, DHHV, float(eps), dtype_code(q), dtype_code(i), state_dtype_code(c_old), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_step")
     return h, (matC_new, vecN_new, scaM_new)
@@ -144,7 +144,7 @@ def mlstm_recurrent_sequence__hip(
     rc = lib.mlstm_hip_recurrent_sequence(
         ptr(qc), ptr(kc), ptr(vc), ptr(ic), ptr(fc), ptr(c), ptr(n), ptr(m),
         ptr(H), ptr(c_out), ptr(n_out), ptr(m_out),
-        B, NH, S, DHQK, DHHV, float(eps), dtype_code(qc), dtype_code(ic), dtype_code(c), current_stream_ptr(dev),
+        B, NH, S, DHQK, DHHV, float(eps), dtype_code(qc), dtype_code(ic), state_dtype_code(c), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_recurrent_sequence")
     if return_last_states:

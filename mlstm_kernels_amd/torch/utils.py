@@ -14,6 +14,13 @@ def dtype_code(t: torch.Tensor) -> int:
     raise TypeError(f"unsupported dtype {t.dtype}: the HIP kernels take float32 or bfloat16 tensors")
 
 
+def state_dtype_code(t: torch.Tensor) -> int:
+    """dtype code of a recurrent state tensor (float32, bfloat16 or float16)."""
+    if t.dtype == torch.float16:
+        return _lib.F16
+    return dtype_code(t)
+
+
 def ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 

@@ -189,56 +189,59 @@ def test_recurrent_sequence_parity(B, NH, T, DQK, DHV, dtype, init):
     assert_state_close(n2, d64(n), 1e-6, "n vs step loop")
 
 
+@pytest.mark.parametrize("sdt,ulp", [(torch.bfloat16, 2.0 ** -7), (torch.float16, 2.0 ** -10)])
 @pytest.mark.parametrize("B,NH,DQK,DHV", [(2, 2, 64, 128), (3, 4, 256, 512), (1, 2, 96, 104), (88, 8, 256, 512),
                                           (162, 8, 256, 512)])
-def test_step_parity_bf16_state(B, NH, DQK, DHV):
-    """States kept in bfloat16 (the reference's dtype_state, triton_step.py:33,67-69): the kernel reads bf16 C, n, m,
-    computes in fp32 and rounds the new states once.  Oracle: the fp64 step on the same bf16-rounded inputs; the new
-    states must lie within one unit in the last place of bfloat16 (at most 2^-7 relative) of the fp64 values, h comes
-    from the unrounded state.  (162, 8, 256, 512) is a 340 MB bf16 state: the streaming variant.)"""
+def test_step_parity_bf16_state(B, NH, DQK, DHV, sdt, ulp):
+    """States kept in bfloat16 or float16 (the reference's dtype_state, triton_step.py:33,67-69): the kernel reads
+    16-bit C, n, m, computes in fp32 and rounds the new states once.  Oracle: the fp64 step on the same rounded
+    inputs; the new states must lie within one unit in the last place of the state type (at most 2^-7 resp. 2^-10
+    relative) of the fp64 values, h comes from the unrounded state.  (162, 8, 256, 512) is a 340 MB state: the
+    streaming variant.)"""
     *_, step, _ = _ops()
     g = torch.Generator().manual_seed(9)
     q, k, v = (torch.randn(B, NH, d, generator=g).bfloat16() for d in (DQK, DQK, DHV))
     i, f = torch.randn(B, NH, 1, generator=g), 3 + torch.randn(B, NH, 1, generator=g)
-    c = torch.randn(B, NH, DQK, DHV, generator=g).bfloat16()
-    n, m = torch.randn(B, NH, DQK, generator=g).bfloat16(), torch.randn(B, NH, 1, generator=g).bfloat16()
+    c = torch.randn(B, NH, DQK, DHV, generator=g).to(sdt)
+    n, m = torch.randn(B, NH, DQK, generator=g).to(sdt), torch.randn(B, NH, 1, generator=g).to(sdt)
     h_r, (c_r, n_r, m_r) = O.recurrent_step(*(d64(t) for t in (q, k, v, i, f, c, n, m)))
-    h, (c2, n2, m2) = step(*(t.to(DEV) for t in (q, k, v, i, f, c, n, m)), dtype_state=torch.bfloat16)
-    assert c2.dtype == n2.dtype == m2.dtype == torch.bfloat16 and h.dtype == torch.bfloat16
+    h, (c2, n2, m2) = step(*(t.to(DEV) for t in (q, k, v, i, f, c, n, m)), dtype_state=sdt)
+    assert c2.dtype == n2.dtype == m2.dtype == sdt and h.dtype == torch.bfloat16
     assert rel_to_scale(h, h_r) <= 5e-3
     for name, x, ref in (("C", c2, c_r), ("n", n2, n_r), ("m", m2, m_r)):
         err = (d64(x) - ref).abs()
         # (+ fp32 rounding of the two products on elements where they nearly cancel)
-        assert bool((err <= 2.0 ** -7 * ref.abs() + 1e-6 * float(ref.abs().max())).all()), (
-            f"{name}: more than one bf16 ulp off (max {float(err.max()):.3e})")
+        assert bool((err <= ulp * ref.abs() + 1e-6 * float(ref.abs().max())).all()), (
+            f"{name}: more than one unit in the last place off (max {float(err.max()):.3e})")
     # in place
     c_dev = c.to(DEV).clone()
     from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_step__hip_fw
     n_new, m_new = torch.empty_like(n2), torch.empty_like(m2)
     h3, (c3, _, _) = mlstm_recurrent_step__hip_fw(c_dev, n.to(DEV), m.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), i.to(DEV),
                                                   f.to(DEV), matC_new=c_dev, vecN_new=n_new, scaM_new=m_new,
-                                                  dtype_state=torch.bfloat16)
+                                                  dtype_state=sdt)
     assert c3.data_ptr() == c_dev.data_ptr() and torch.equal(c3, c2) and torch.equal(h3, h)
 
 
+@pytest.mark.parametrize("sdt,ulp", [(torch.bfloat16, 2.0 ** -7), (torch.float16, 2.0 ** -10)])
 @pytest.mark.parametrize("B,NH,T,DQK,DHV", [(2, 2, 9, 64, 128), (3, 4, 33, 256, 512), (1, 2, 5, 96, 100), (1, 1, 4, 384, 64)])
-def test_recurrent_sequence_bf16_state(B, NH, T, DQK, DHV):
-    """bf16 states in and out of the multi-token kernel: fp32 between the tokens, rounded once at the end."""
+def test_recurrent_sequence_bf16_state(B, NH, T, DQK, DHV, sdt, ulp):
+    """16-bit states in and out of the multi-token kernel: fp32 between the tokens, rounded once at the end."""
     *_, seq = _ops()
     g = torch.Generator().manual_seed(13)
     q, k, v = (torch.randn(B, NH, T, d, generator=g).bfloat16() for d in (DQK, DQK, DHV))
     i, f = torch.randn(B, NH, T, generator=g), 3 + torch.randn(B, NH, T, generator=g)
-    c0 = torch.randn(B, NH, DQK, DHV, generator=g).bfloat16()
-    n0, m0 = torch.randn(B, NH, DQK, generator=g).bfloat16(), torch.randn(B, NH, 1, generator=g).bfloat16()
+    c0 = torch.randn(B, NH, DQK, DHV, generator=g).to(sdt)
+    n0, m0 = torch.randn(B, NH, DQK, generator=g).to(sdt), torch.randn(B, NH, 1, generator=g).to(sdt)
     H_r, (c_r, n_r, m_r) = O.recurrent_sequence(*(d64(t) for t in (q, k, v, i, f)), c_initial=d64(c0), n_initial=d64(n0),
                                                 m_initial=d64(m0))
     H, (c2, n2, m2) = seq(*(t.to(DEV) for t in (q, k, v, i, f)), c_initial=c0.to(DEV), n_initial=n0.to(DEV),
-                          m_initial=m0.to(DEV), return_last_states=True, dtype_state=torch.bfloat16)
-    assert c2.dtype == n2.dtype == m2.dtype == torch.bfloat16
+                          m_initial=m0.to(DEV), return_last_states=True, dtype_state=sdt)
+    assert c2.dtype == n2.dtype == m2.dtype == sdt
     assert rel_to_scale(H, H_r) <= 5e-3
     for name, x, ref in (("C", c2, c_r), ("n", n2, n_r), ("m", m2, m_r)):
         err = (d64(x) - ref).abs()
-        assert bool((err <= 2.0 ** -7 * ref.abs() + 1e-5 * float(ref.abs().max())).all()), f"{name}: max error {float(err.max()):.3e}"
+        assert bool((err <= ulp * ref.abs() + 1e-5 * float(ref.abs().max())).all()), f"{name}: max error {float(err.max()):.3e}"
 
 
 def test_recurrent_sequence_rejects_bad_arguments():
