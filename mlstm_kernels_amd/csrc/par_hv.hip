@@ -63,7 +63,6 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
   uint16_t* Ts = Ps + 64 * PS;
   constexpr int t_region = (128 * KS > VR * VS) ? 128 * KS : VR * VS;
   static_assert(VR >= 16 && VR <= 128, "value slabs hold 16 to 128 rows");
-  static_assert(t_region >= 32 * HS, "the slab buffer also stages 32 output rows");
   float* nvec = (float*)(Ts + t_region);  // [64] gate vector of this workgroup's positions: u_t (forward) / w_j (dV)
   float* ovec = nvec + 64;              // [128] gate vector of the source chunk: w_j (forward) / u_t (dV)
   float* orho = ovec + 128;             // [128] dV: rho_t of the source chunk
@@ -582,15 +581,19 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
         }
       }
     }
-    // ---- epilogue: (normalise,) round, transpose through the slab buffer (32 positions at a time), coalesced store
+    // ---- epilogue: (normalise,) round, transpose through LDS, coalesced store.  The score block and the slab buffer
+    // are both free now and lie next to each other: together they hold all 64 positions of a column tile, so a tile
+    // costs two barriers.
+    static_assert(64 * PS + t_region >= 64 * HS, "score block + slab buffer stage 64 output rows");
+    uint16_t* const Os = Ps;
 #pragma unroll
     for (int tl = 0; tl < NTG; ++tl) {
       uint16_t* Og = a.Out + (size_t)bh * S * DHHV + grp * GW + tl * WT;
+      const int le = opaque(lane);
+      const int r = le & 31, h = le >> 5;
+      __syncthreads();  // staging area free (last value slab and score block consumed / previous tile stored; inv written)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        const int le = opaque(lane);
-        const int r = le & 31, h = le >> 5;
-        __syncthreads();  // slab buffer free (last value slab consumed / previous half stored; inv written)
         const float iv = IS_DV ? 1.f : (normed ? osc[nb] : inv[32 * nb + r]);
         const float sh = normed ? osh[nb] : 0.f;
 #pragma unroll
@@ -598,18 +601,18 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
 #pragma unroll
           for (int g4 = 0; g4 < 4; ++g4) {
             const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
-            *(uint2*)(Ts + r * HS + w0) =
+            *(uint2*)(Os + (32 * nb + r) * HS + w0) =
                 make_uint2(pack_bf16x2(acc[tl][mb][nb][4 * g4 + 0] * iv + sh, acc[tl][mb][nb][4 * g4 + 1] * iv + sh),
                            pack_bf16x2(acc[tl][mb][nb][4 * g4 + 2] * iv + sh, acc[tl][mb][nb][4 * g4 + 3] * iv + sh));
           }
-        __syncthreads();
-        constexpr int vec_per_row = WT / 8;
-        for (int idx = opaque(tid); idx < 32 * vec_per_row; idx += NTH) {
-          const int j = idx / vec_per_row, cv = idx % vec_per_row;
-          const int t = t_base + n0 + 32 * nb + j;
-          // non-temporal: nobody in this launch reads the output, it should not evict shared operands from the L2
-          if (t < S) __builtin_nontemporal_store(*(const u32x4*)(Ts + j * HS + cv * 8), (u32x4*)(Og + (size_t)t * DHHV + cv * 8));
-        }
+      }
+      __syncthreads();
+      constexpr int vec_per_row = WT / 8;
+      for (int idx = opaque(tid); idx < 64 * vec_per_row; idx += NTH) {
+        const int j = idx / vec_per_row, cv = idx % vec_per_row;
+        const int t = t_base + n0 + j;
+        // non-temporal: nobody in this launch reads the output, it should not evict shared operands from the L2
+        if (t < S) __builtin_nontemporal_store(*(const u32x4*)(Os + j * HS + cv * 8), (u32x4*)(Og + (size_t)t * DHHV + cv * 8));
       }
     }
   }
