@@ -77,6 +77,33 @@ def test_shape_rules_of_the_xl_chunk_operator():
         validate_xl_chunk_shapes(384, 256)      # not divisible by the chunk size
 
 
+def test_operator_options_are_validated_on_the_host():
+    """The options this package adds to or honours from the reference's keyword set: chunk_size_intra -> state stride
+    (mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:118-121), kernel path, head norm, state dtype."""
+    from mlstm_kernels_amd.torch.chunkwise.hip_xl_chunk import _state_stride
+    from mlstm_kernels_amd.torch.recurrent.hip_step import _check_state_dtype
+
+    assert _state_stride({}, "op") == 0                                   # library default
+    assert _state_stride({"chunk_size_intra": 128}, "op") == 1
+    assert _state_stride({"chunk_size_inter": 128, "chunk_size_intra": 512}, "op") == 4
+    assert _state_stride({"siz_b_L_parallel": 64, "num_warps_intra": 4, "recompute_states_in_bw": True}, "op") == 0
+    for bad in ({"chunk_size_inter": 64}, {"chunk_size_intra": 192}, {"chunk_size_intra": 2048}, {"chunk_size_intra": 0}):
+        with pytest.raises(ValueError):
+            _state_stride(bad, "op")
+    with pytest.raises(TypeError, match="unexpected keyword"):
+        _state_stride({"chunk_size_itnra": 256}, "op")
+    assert [_lib.path_code(n) for n in ("auto", "split", "fused")] == [_lib.PATH_AUTO, _lib.PATH_SPLIT, _lib.PATH_FUSED]
+    with pytest.raises(ValueError):
+        _lib.path_code("triton")
+    assert [_lib.norm_code(n) for n in ("none", "layer", "rms")] == [_lib.NORM_NONE, _lib.NORM_LAYER, _lib.NORM_RMS]
+    with pytest.raises(ValueError):
+        _lib.norm_code("group")
+    for ok in (torch.float32, torch.bfloat16, torch.float16):
+        assert _check_state_dtype(ok) is ok
+    with pytest.raises(NotImplementedError):
+        _check_state_dtype(torch.float64)
+
+
 def test_hip_kernels_have_no_cpu_fallback():
     q, k, v, i, f = make_qkvif(1, 1, 128, 64, 64)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
