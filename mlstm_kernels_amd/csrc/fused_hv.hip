@@ -585,13 +585,13 @@ const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_
   if (a.stride < 1 || a.stride > kMaxStateStride) return "fused_hv: state stride out of range";
   // one wave per 32-position block (four waves, one per SIMD): the eight-wave form, in which the two waves of a block
   // both compute its scores, was measured slower
-  constexpr int MLSTM_FUSED_NWQ = 1;
+  constexpr int kWavesPerBlock = 1;
   if (is_dv) {
-    if (a.DHQK == 256) return launch_fused_hv_t<256, true, false, MLSTM_FUSED_NWQ>(a, BH, stream);
-    return launch_fused_hv_t<128, true, false, MLSTM_FUSED_NWQ>(a, BH, stream);
+    if (a.DHQK == 256) return launch_fused_hv_t<256, true, false, kWavesPerBlock>(a, BH, stream);
+    return launch_fused_hv_t<128, true, false, kWavesPerBlock>(a, BH, stream);
   }
-  if (a.DHQK == 256) return launch_fused_hv_t<256, false, true, MLSTM_FUSED_NWQ>(a, BH, stream);
-  return launch_fused_hv_t<128, false, true, MLSTM_FUSED_NWQ>(a, BH, stream);
+  if (a.DHQK == 256) return launch_fused_hv_t<256, false, true, kWavesPerBlock>(a, BH, stream);
+  return launch_fused_hv_t<128, false, true, kWavesPerBlock>(a, BH, stream);
 }
 
 }  // namespace mlstm
