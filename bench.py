@@ -283,6 +283,7 @@ def main():
     for name, entry in kernels.items():
         if name in traffic:
             entry["hbm_bytes_measured"] = traffic[name]
+            entry["measured_gbs"] = round(traffic[name] / (entry["avg_ms"] * 1e-3) / 1e9, 1)   # rocprofv3 bytes / this run's time
 
     extra = {}
     if not args.no_extra:
