@@ -275,7 +275,9 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   sa.stride = stride;
   {
     ProfileScope ps("scan_fw", st);
-    if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/true, st)) return fail(e);
+    // The bf16 head + remainder split of the value operand only serves the fp32 last state (1e-5 instead of 1.5e-3
+    // relative); the chunk states are rounded to bf16 anyway, so a call that returns no last state skips it.
+    if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/c_last != nullptr, st)) return fail(e);
   }
   if (check_launch("scan_fw")) return 1;
 

