@@ -137,6 +137,9 @@ size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, in
  *   c0,n0,m0: initial states or NULL (all three NULL together; m0 ignored for the sig gate).
  *   H (B,NH,S,DHHV) in dtype_qkv.  n_out, m_out: optional fp32 (B,NH,S) per-row normaliser max(|den|,floor)
  *   and stabiliser (NULL to skip).  c_last,n_last,m_last: optional fp32 last states (NULL to skip).
+ *   With c_last given, the state scan carries the gated values as a bf16 head plus a bf16 remainder, so c_last is
+ *   accurate to ~1e-5 relative; with c_last NULL it rounds them to bf16 once (as the replaced kernels do), which is
+ *   a fifth faster and changes H only within its bf16 tolerance.
  *   normalize applies to the sig gate only (0: H is the bare numerator).
  */
 int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const void* i, const void* f,
