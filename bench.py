@@ -24,7 +24,7 @@ Objects on the JSON line besides the contract's keys:
   decode_step   -- fused decode step at B=256 after a chunkwise prefill of 2048 positions: ms per step, algorithmic
                    GB/s, its own HBM roofline; B=64 and B=16 (whose state fits the memory-side cache: "bound": "mall");
                    multi_token: 128 tokens per (batch, head) in ONE launch of the multi-token kernel.
-  extra         -- the other BASELINE configurations, same protocol: B=16/S=4096 and B=64/S=1024 (fwd+bwd), the
+  extra         -- the other benchmark configurations of the reference, same protocol: B=16/S=4096 and B=64/S=1024 (fwd+bwd), the
                    sigmoid gate with a non-zero initial state at B=4/S=16384, forward-only at B=4/S=16384, and the
                    latter two shapes with the multi-head layer norm fused into the output kernel.
   cpu_baseline  -- the fp32 PyTorch oracle (restatement of the reference's native chunkwise forward + custom backward)
@@ -160,7 +160,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configurations and the small decode batches")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations and the small decode batches")
     ap.add_argument("--state-stride", type=int, default=0, help="chunk states kept every n-th chunk (0 = library default)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -75,7 +75,7 @@ def case(fw, bw, seed, B, NH, S, DQK, DHV, L, init, dcl):
 def main():
     fw, bw = load_native()
     cases = {
-        "a": case(fw, bw, 0, 1, 2, 256, 64, 64, 64, False, False),    # BASELINE config-1 shape, zero initial state
+        "a": case(fw, bw, 0, 1, 2, 256, 64, 64, 64, False, False),    # the small fp32 shape, zero initial state
         "b": case(fw, bw, 1, 1, 2, 128, 64, 128, 32, True, True),     # initial states and an upstream dC_last
     }
     flat = {}

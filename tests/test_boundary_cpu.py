@@ -141,7 +141,7 @@ def test_library_exports_every_declared_symbol():
     assert rc != 0 and b"null pointer" in lib.mlstm_hip_last_error()
 
 
-# ------------------------------------------------------------------ BASELINE config 1: CPU plumbing check
+# ------------------------------------------------------------------ the small fp32 shape: CPU plumbing check
 def test_backend_module_train_mode_cpu_plumbing():
     # B=1, NH=4, S=256, DHQK=64, DHHV=64, chunk_size=64, fp32, zero initial states, return_last_states=True
     q, k, v, i, f = make_qkvif(1, 4, 256, 64, 64, seed=0, dtype=torch.float32)

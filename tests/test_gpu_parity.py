@@ -262,7 +262,7 @@ def test_recurrent_sequence_rejects_bad_arguments():
 
 @pytest.mark.parametrize("B", [16, 64, 256])
 def test_decode_after_prefill(B):
-    """BASELINE config 5: prefill S=2048 with the chunkwise kernel, then 128 consecutive decode steps (state updated
+    """The reference's decode benchmark: prefill S=2048 with the chunkwise kernel, then 128 consecutive decode steps (state updated
     in place) at B = 16, 64 and 256 (the last one streams its 1 GiB state past the caches with the non-temporal
     kernel variant); the oracle does the same in fp64 for the first and the last batch row.  Inputs are drawn on the
     GPU (the full-batch tensors are too large to draw on the host) and the checked rows are copied out."""
@@ -343,8 +343,8 @@ def test_decode_steps_in_hip_graph():
 
 # ------------------------------------------------------------------------------------------ chunkwise forward
 @pytest.mark.parametrize("cfg", [
-    dict(B=1, NH=4, S=256, DQK=64, DHV=64, L=64, seed=0, dtype=torch.float32),    # BASELINE config 1 shape
-    dict(B=2, NH=4, S=512, DQK=128, DHV=256, L=256, seed=1, dtype=torch.bfloat16),  # BASELINE config 2
+    dict(B=1, NH=4, S=256, DQK=64, DHV=64, L=64, seed=0, dtype=torch.float32),    # the reference suite's small fp32 shape
+    dict(B=2, NH=4, S=512, DQK=128, DHV=256, L=256, seed=1, dtype=torch.bfloat16),  # the reference suite's bf16 shape
     dict(B=1, NH=2, S=144, DQK=64, DHV=128, L=16, seed=2, dtype=torch.bfloat16),   # ragged tail (128 + 16)
     dict(B=1, NH=2, S=32, DQK=64, DHV=64, L=32, seed=3, dtype=torch.bfloat16),     # shorter than one chunk
     dict(B=1, NH=1, S=256, DQK=512, DHV=1024, L=128, seed=4, dtype=torch.bfloat16),  # several head-dim / value tiles
@@ -471,7 +471,7 @@ def test_chunkwise_fwbw_small(kw):
 
 @pytest.mark.parametrize("B,S", [(64, 1024), (16, 4096), (4, 16384)])
 def test_chunkwise_fwbw_xlstm7b_shape_exp(B, S):
-    """BASELINE config 3: NH=8, DHQK=256, DHHV=512, B*S = 65536, upstream dH ~ N(0,1).  The whole tensor runs on
+    """The reference's headline benchmark shape (xLSTM-7B heads): NH=8, DHQK=256, DHHV=512, B*S = 65536, upstream dH ~ N(0,1).  The whole tensor runs on
     the GPU; two (batch, head) pairs are checked against the fp64 oracle over the full sequence."""
     _fwbw_case(B, 8, S, 256, 512, seed=0, pairs=[(0, 0), (B - 1, 7)])   # first and last workgroups of every launch
 
@@ -482,7 +482,7 @@ def test_chunkwise_fwbw_xlstm7b_shape_training_call():
 
 
 def test_chunkwise_fwbw_xlstm7b_shape_sig():
-    """BASELINE config 4: mLSTMsig, B=4, S=16384, non-zero initial C ~ N(0,0.1), n ~ N(0,0.1), m = 0."""
+    """The reference's sigmoid-gate benchmark shape: mLSTMsig, B=4, S=16384, non-zero initial C ~ N(0,0.1), n ~ N(0,0.1), m = 0."""
     _fwbw_case(4, 8, 16384, 256, 512, siging=True, init=True, seed=0, pairs=[(1, 4), (2, 3)])   # middle of the grid
 
 
