@@ -25,8 +25,9 @@ Objects on the JSON line besides the contract's keys:
                    GB/s, its own HBM roofline; B=64 and B=16 (whose state fits the memory-side cache: "bound": "mall");
                    multi_token: 128 tokens per (batch, head) in ONE launch of the multi-token kernel.
   extra         -- the other benchmark configurations of the reference, same protocol: B=16/S=4096 and B=64/S=1024 (fwd+bwd), the
-                   sigmoid gate with a non-zero initial state at B=4/S=16384, forward-only at B=4/S=16384, and the
-                   latter two shapes with the multi-head layer norm fused into the output kernel.
+                   sigmoid gate with a non-zero initial state at B=4/S=16384, float16 operands at B=4/S=16384,
+                   forward-only at B=4/S=16384 (without and with the last states returned), and the forward and the
+                   forward+backward with the multi-head layer norm fused into the output kernel.
   cpu_baseline  -- the fp32 PyTorch oracle (restatement of the reference's native chunkwise forward + custom backward)
                    timed on this box's host cores on the same workload, plus the oracle's decode step.
 
@@ -186,16 +187,17 @@ def main():
     intra = {} if args.state_stride == 0 else {"chunk_size_intra": CHUNK * args.state_stride}
     stride = args.state_stride or _lib.default_state_stride(B, NH, S, DHQK, DHHV)
 
-    def run_config(Bc, Sc, steps, warmup, sig=False, init=False, backward=True, profile_steps=3, head_norm="none"):
+    def run_config(Bc, Sc, steps, warmup, sig=False, init=False, backward=True, profile_steps=3, head_norm="none",
+                   dtype=torch.bfloat16, last_states=False):
         """Times `steps` passes of one configuration (median of per-step HIP-event times, caches flushed before every
         step), then profiles `profile_steps` further passes kernel by kernel."""
-        q = rn(Bc, NH, Sc, DHQK).bfloat16().requires_grad_(backward)
-        k = rn(Bc, NH, Sc, DHQK).bfloat16().requires_grad_(backward)
-        v = rn(Bc, NH, Sc, DHHV).bfloat16().requires_grad_(backward)
+        q = rn(Bc, NH, Sc, DHQK).to(dtype).requires_grad_(backward)
+        k = rn(Bc, NH, Sc, DHQK).to(dtype).requires_grad_(backward)
+        v = rn(Bc, NH, Sc, DHHV).to(dtype).requires_grad_(backward)
         i = rn(Bc, NH, Sc).requires_grad_(backward)
         f = (3 + rn(Bc, NH, Sc)).requires_grad_(backward)
-        dH = rn(Bc, NH, Sc, DHHV).bfloat16()
-        kw = dict(chunk_size=CHUNK, autocast_kernel_dtype=torch.bfloat16, head_norm=head_norm, **intra)
+        dH = rn(Bc, NH, Sc, DHHV).to(dtype)
+        kw = dict(chunk_size=CHUNK, autocast_kernel_dtype=dtype, head_norm=head_norm, return_last_states=last_states, **intra)
         if init:
             kw.update(c_initial=0.1 * rn(Bc, NH, DHQK, DHHV), n_initial=0.1 * rn(Bc, NH, DHQK),
                       m_initial=torch.zeros(Bc, NH, 1, device=dev))
@@ -203,7 +205,8 @@ def main():
 
         def step():
             if backward:
-                op(q, k, v, i, f, **kw).backward(dH)
+                out = op(q, k, v, i, f, **kw)
+                (out[0] if last_states else out).backward(dH)
             else:
                 with torch.no_grad():
                     op(q, k, v, i, f, **kw)
@@ -290,7 +293,9 @@ def main():
         n_extra = max(5, args.steps // 2)
         for tag, cfg in (("exp_fwbw_B16_S4096", dict(Bc=16, Sc=4096)), ("exp_fwbw_B64_S1024", dict(Bc=64, Sc=1024)),
                          ("sig_fwbw_B4_S16384_init", dict(Bc=4, Sc=16384, sig=True, init=True)),
+                         ("exp_fwbw_B4_S16384_float16", dict(Bc=4, Sc=16384, dtype=torch.float16)),
                          ("exp_fw_B4_S16384", dict(Bc=4, Sc=16384, backward=False)),
+                         ("exp_fw_B4_S16384_last_states", dict(Bc=4, Sc=16384, backward=False, last_states=True)),
                          ("exp_fw_B4_S16384_head_norm_layer", dict(Bc=4, Sc=16384, backward=False, head_norm="layer")),
                          ("exp_fwbw_B4_S16384_head_norm_layer", dict(Bc=4, Sc=16384, head_norm="layer"))):
             r = run_config(steps=n_extra, warmup=2, **cfg)

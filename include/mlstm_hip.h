@@ -10,8 +10,11 @@
  *     C (B,NH,DHQK,DHHV) fp32; n (B,NH,DHQK) fp32; m (B,NH) fp32.
  *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it.
  *   - Return value 0 = success; anything else = failure, message via mlstm_hip_last_error().
- *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1 (and MLSTM_F16 = 2 for the recurrent states only).  gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp),
- *     MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
+ *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1, MLSTM_F16 = 2.  The chunkwise entry points take q/k/v (and dH) in
+ *     bf16 or fp16 and multiply in that format on the matrix cores with fp32 accumulation (the kept chunk states are
+ *     rounded to the same format; fp16 has three more mantissa bits and overflows above 65504); gates in fp32, bf16 or
+ *     fp16.  The decode entry points take q/k/v and gates in fp32 or bf16 and states in fp32, bf16 or fp16.
+ *   - gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp), MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
  *   - Supported shapes: DHQK % 64 == 0 (at most 896), DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
  *
  * Each entry point names the reference interface it replaces (paths relative to the reference checkout).
@@ -28,7 +31,7 @@ extern "C" {
 
 #define MLSTM_F32 0
 #define MLSTM_BF16 1
-#define MLSTM_F16 2 /* recurrent states only (dtype_state) */
+#define MLSTM_F16 2
 #define MLSTM_GATE_EXP 0
 #define MLSTM_GATE_SIG 1
 
@@ -137,9 +140,10 @@ size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, in
  *   c0,n0,m0: initial states or NULL (all three NULL together; m0 ignored for the sig gate).
  *   H (B,NH,S,DHHV) in dtype_qkv.  n_out, m_out: optional fp32 (B,NH,S) per-row normaliser max(|den|,floor)
  *   and stabiliser (NULL to skip).  c_last,n_last,m_last: optional fp32 last states (NULL to skip).
- *   With c_last given, the state scan carries the gated values as a bf16 head plus a bf16 remainder, so c_last is
- *   accurate to ~1e-5 relative; with c_last NULL it rounds them to bf16 once (as the replaced kernels do), which is
- *   a fifth faster and changes H only within its bf16 tolerance.
+ *   With c_last given, the state scan carries the gated values as a 16-bit head plus a 16-bit remainder, so c_last
+ *   is accurate to ~1e-5 relative; with c_last NULL it rounds them once (as the replaced kernels do), which is a
+ *   fifth faster and changes H only within the tolerance of its 16-bit operands.
+ *   MLSTM_PATH_FUSED takes bf16 only.
  *   normalize applies to the sig gate only (0: H is the bare numerator).
  */
 int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const void* i, const void* f,
@@ -155,7 +159,7 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
  * Backward of the fused head norm: dX = rstd * (dY - mean_D(dY) - Y * mean_D(dY * Y)) for MLSTM_NORM_LAYER,
  * dX = rstd * (dY - Y * mean_D(dY * Y)) for MLSTM_NORM_RMS, per row of D = 64, 128, 256 or 512 values.
  * Replaces the autograd backward of the reference's layer_normalize / rms_normalize
- * (mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-35).  dY, Y, dX: (rows, D) in dtype (bf16);
+ * (mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-35).  dY, Y, dX: (rows, D) in dtype (bf16 or fp16);
  * rstd: (rows) fp32 as written by the forward.
  */
 int mlstm_hip_head_norm_bw(const void* dY, const void* Y, const float* rstd, void* dX, size_t rows, int D,

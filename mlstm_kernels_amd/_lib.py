@@ -10,7 +10,7 @@ _lock = threading.Lock()
 _lib = None
 
 F32, BF16 = 0, 1
-F16 = 2  # recurrent states only (dtype_state)
+F16 = 2
 GATE_EXP, GATE_SIG = 0, 1
 PATH_AUTO, PATH_SPLIT, PATH_FUSED = 0, 1, 2
 NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2

@@ -196,13 +196,15 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   if (!q || !k || !v || !i || !f || !H || !workspace) return failw("null pointer argument");
   if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return failw(e);
   if (const char* e = check_options(path, state_stride, DHQK, DHHV)) return failw(e);
-  if (dtype_qkv != MLSTM_BF16) return failw("q/k/v must be bf16");
-  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return failw("unsupported gate dtype");
+  if (dtype_qkv != MLSTM_BF16 && dtype_qkv != MLSTM_F16) return failw("q/k/v must be bf16 or fp16");
+  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16 && dtype_gates != MLSTM_F16) return failw("unsupported gate dtype");
+  const int f16 = dtype_qkv == MLSTM_F16;
   if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return failw("unknown gate code");
   const bool has_c0 = c0 != nullptr;
   if (has_c0 != (n0 != nullptr)) return failw("c0 and n0 must be given together");
   if (gate == MLSTM_GATE_EXP && has_c0 != (m0 != nullptr)) return failw("initial states must be given together");
   const bool fused = use_fused(path, DHQK, DHHV);
+  if (fused && f16) return failw("the fused kernel path multiplies bf16 operands only");
   if (head_norm != MLSTM_NORM_NONE) {
     if (head_norm != MLSTM_NORM_LAYER && head_norm != MLSTM_NORM_RMS) return failw("unknown head norm code");
     if (fused) return failw("the fused kernel path has no head norm epilogue");
@@ -273,6 +275,7 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   sa.eps = eps;
   sa.backward = 0;
   sa.stride = stride;
+  sa.f16 = f16;
   {
     ProfileScope ps("scan_fw", st);
     // The bf16 head + remainder split of the value operand only serves the fp32 last state (1e-5 instead of 1.5e-3
@@ -296,6 +299,7 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   pa.use_nrow = !(sig && !normalize);
   pa.stride = stride;
   pa.head_norm = head_norm;
+  pa.f16 = f16;
   pa.norm_eps = norm_eps;
   pa.norm_mean = norm_mean;
   pa.norm_rstd = norm_rstd;
@@ -325,10 +329,11 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
 int mlstm_hip_head_norm_bw(const void* dY, const void* Y, const float* rstd, void* dX, size_t rows, int D, int head_norm,
                            int dtype, void* stream) {
   if (!dY || !Y || !rstd || !dX) return fail("mlstm_hip_head_norm_bw: null pointer argument");
-  if (dtype != MLSTM_BF16) return fail("mlstm_hip_head_norm_bw: rows must be bf16");
+  if (dtype != MLSTM_BF16 && dtype != MLSTM_F16) return fail("mlstm_hip_head_norm_bw: rows must be bf16 or fp16");
   mlstm::HeadNormBwArgs a;
   a.dY = (const uint16_t*)dY; a.Y = (const uint16_t*)Y; a.rstd = rstd; a.dX = (uint16_t*)dX;
   a.rows = rows; a.D = D; a.kind = head_norm;
+  a.f16 = dtype == MLSTM_F16;
   {
     ProfileScope ps("head_norm_bw", (hipStream_t)stream);
     if (const char* e = mlstm::launch_head_norm_bw(a, (hipStream_t)stream)) return fail(e);
@@ -352,8 +357,10 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
     return fail("mlstm_hip_chunkwise_bw: null pointer argument");
   if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return fail(e);
   if (const char* e = check_options(path, state_stride, DHQK, DHHV)) return fail(e);
-  if (dtype_qkv != MLSTM_BF16) return fail("mlstm_hip_chunkwise_bw: q/k/v/dH must be bf16");
-  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) return fail("mlstm_hip_chunkwise_bw: unsupported gate dtype");
+  if (dtype_qkv != MLSTM_BF16 && dtype_qkv != MLSTM_F16) return fail("mlstm_hip_chunkwise_bw: q/k/v/dH must be bf16 or fp16");
+  if (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16 && dtype_gates != MLSTM_F16)
+    return fail("mlstm_hip_chunkwise_bw: unsupported gate dtype");
+  const int f16 = dtype_qkv == MLSTM_F16;
   if (gate != MLSTM_GATE_EXP && gate != MLSTM_GATE_SIG) return fail("mlstm_hip_chunkwise_bw: unknown gate code");
   const int stride = resolve_stride(state_stride);
   const int tiles = DHQK / mlstm::par_qk_head_tile(DHQK);
@@ -368,6 +375,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   const float qk_scale = 1.0f / sqrtf((float)DHQK);
 
   if (use_fused(path, DHQK, DHHV)) {
+    if (f16) return fail("mlstm_hip_chunkwise_bw: the fused kernel path multiplies bf16 operands only");
     mlstm::FusedHvArgs fa;
     memset(&fa, 0, sizeof(fa));
     fa.Q = (const uint16_t*)q; fa.K = (const uint16_t*)k; fa.V = (const uint16_t*)v; fa.dH = (const uint16_t*)dH;
@@ -401,6 +409,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
     sa.qk_scale = qk_scale; sa.eps = eps;
     sa.backward = 1;
     sa.stride = stride;
+    sa.f16 = f16;
     {
       ProfileScope ps("scan_bw", st);
       if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/false, st)) return fail(e);
@@ -418,6 +427,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
     pv.qk_scale = qk_scale; pv.eps = eps;
     pv.sig_gate = sig; pv.use_nrow = use_nrow;
     pv.stride = stride;
+    pv.f16 = f16;
     {
       ProfileScope ps("par_dv", st);
       if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
@@ -434,6 +444,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   pq.qk_scale = qk_scale; pq.eps = eps;
   pq.use_nrow = use_nrow;
   pq.stride = stride;
+  pq.f16 = f16;
   // dQ and dK in one launch: the workgroups of a chunk run side by side and share the Q, K, V and dH rows they stream
   pq.states = ws.cstates; pq.Out = (uint16_t*)dQ; pq.rowdot = bws.qdq;
   pq.states2 = bws.dcstates; pq.Out2 = (uint16_t*)dK; pq.rowdot2 = bws.kdk;

@@ -17,10 +17,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 // is promoted to registers (struct copies become memcpy calls the optimiser leaves in scratch memory)
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// 8 bf16 as raw bits; convertible to the MFMA operand type without data movement
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+// 8 bf16 (or fp16) as raw bits; convertible to the MFMA operand type without data movement
 union Frag {
   uint4 u;
   bf16x8 v;
+  f16x8 hv;
   uint16_t h[8];
   uint32_t w[4];
   uint2 d[2];
@@ -51,6 +53,45 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // acc[i] = D[8*(i/4) + 4h + (i%4)][r].
 __device__ __forceinline__ void mfma32(f32x16& acc, const Frag& a, const Frag& b) {
   acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
+}
+
+
+// The chunkwise kernels multiply either bfloat16 (F16 = false) or float16 (F16 = true) operands; the accumulators,
+// gates, normalisers and row scales are fp32 either way.  Element helpers for both 16-bit formats:
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+template <bool F16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {  // two fp32 -> one packed pair, round to nearest even
+  if constexpr (F16) {
+    const f16x2 hv = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, hv);
+  } else {
+    return pack_bf16x2(lo, hi);
+  }
+}
+template <bool F16>
+__device__ __forceinline__ float lo2(uint32_t w) {  // low element of a packed pair
+  if constexpr (F16) return (float)__builtin_bit_cast(f16x2, w)[0];
+  else return __uint_as_float(w << 16);
+}
+template <bool F16>
+__device__ __forceinline__ float hi2(uint32_t w) {  // high element of a packed pair
+  if constexpr (F16) return (float)__builtin_bit_cast(f16x2, w)[1];
+  else return __uint_as_float(w & 0xffff0000u);
+}
+template <bool F16>
+__device__ __forceinline__ float elem_to_f32(uint16_t b) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, b);
+  else return bf16_bits_to_f32(b);
+}
+template <bool F16>
+__device__ __forceinline__ uint16_t f32_to_elem(float x) {
+  if constexpr (F16) return __builtin_bit_cast(uint16_t, (_Float16)x);
+  else return f32_to_bf16_bits(x);
+}
+template <bool F16>
+__device__ __forceinline__ void mfma32(f32x16& acc, const Frag& a, const Frag& b) {
+  if constexpr (F16) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a.hv, b.hv, acc, 0, 0, 0);
+  else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc, 0, 0, 0);
 }
 
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -89,12 +130,14 @@ __device__ __forceinline__ float log_sigmoid(float x) {
   return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
+// dtype: 0 float32, 1 bfloat16, 2 float16
 __device__ __forceinline__ float load_scalar(const void* p, size_t idx, int dtype) {
-  return dtype == 0 ? ((const float*)p)[idx] : bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+  if (dtype == 0) return ((const float*)p)[idx];
+  if (dtype == 1) return bf16_bits_to_f32(((const uint16_t*)p)[idx]);
+  return (float)((const _Float16*)p)[idx];
 }
 
 // Recurrent states may be kept in float32 (0), bfloat16 (1) or float16 (2); the arithmetic is float32.
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float load_state_scalar(const void* p, size_t idx, int sdt) {
   if (sdt == 0) return ((const float*)p)[idx];
   if (sdt == 1) return bf16_bits_to_f32(((const uint16_t*)p)[idx]);

@@ -10,8 +10,8 @@
 namespace mlstm {
 
 struct ScanArgs {
-  const uint16_t* X;      // (B,NH,S,DHQK) bf16: K (forward) or Q (backward)
-  const uint16_t* Y;      // (B,NH,S,DHHV) bf16: V (forward) or dH (backward)
+  const uint16_t* X;      // (B,NH,S,DHQK) bf16/fp16: K (forward) or Q (backward)
+  const uint16_t* Y;      // (B,NH,S,DHHV) bf16/fp16: V (forward) or dH (backward)
   const float* scale_a;   // [BH][Sp] forward: abar; backward: bbar
   const float* nrow;      // backward: [BH][Sp] row normaliser or nullptr; forward: nullptr
   const float* gbar;      // [BH][NC]
@@ -25,6 +25,7 @@ struct ScanArgs {
   float qk_scale, eps;
   int backward;
   int stride;             // a chunk state is kept every `stride` chunks
+  int f16;                // X, Y and the state fragments are float16 instead of bfloat16
 };
 
 struct ParHvArgs {
@@ -46,6 +47,7 @@ struct ParHvArgs {
   float norm_eps;
   float* norm_mean;         // forward with head_norm: (B,NH,S) row means (0 for rms)
   float* norm_rstd;         // forward with head_norm: (B,NH,S) reciprocal standard deviations
+  int f16;                  // inputs, state fragments and Out are float16 instead of bfloat16
 };
 
 struct HeadNormBwArgs {
@@ -55,6 +57,7 @@ struct HeadNormBwArgs {
   uint16_t* dX;             // (rows, D) bf16 gradient of the input of the norm
   size_t rows;
   int D, kind;              // kind: 1 layer norm, 2 rms norm
+  int f16;                  // dY, Y and dX are float16 instead of bfloat16
 };
 
 struct FusedHvArgs {
@@ -91,6 +94,7 @@ struct ParQkArgs {
   float qk_scale, eps;
   int use_nrow;
   int stride;               // a chunk state is kept every `stride` chunks
+  int f16;                  // inputs, state fragments and outputs are float16 instead of bfloat16
 };
 
 struct GateGradArgs {

@@ -43,7 +43,7 @@ namespace mlstm {
 // PD = how many contraction steps ahead the state fragments are fetched (must divide DHQK / 16).
 // MW = value columns per wave (64 or 32): WT / MW waves share a tile.  NTG = column tiles per group (1 or 2).
 #define PAR_HV_WPE(WT_, MW_) ((WT_) / (MW_) >= 8 ? 4 : ((WT_) >= 128 ? 2 : 1))
-template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM>
+template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM, bool F16>
 __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId blk) {
   constexpr int NWAVE = WT / MW;   // each wave owns MW value columns of every tile of the group = MB MFMA row blocks
   constexpr int MB = MW / 32;
@@ -298,7 +298,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
           Frag A, B;                                                                                                 \
           A.u = *(const uint4*)(Ts + (32 * obc + r) * KS + 16 * ds + 8 * h);                                         \
           B.u = *(const uint4*)(Ns + (32 * nb + r) * QS + (ks_) * 64 + 16 * ds + 8 * h);                             \
-          mfma32(sacc[k], A, B);                                                                                     \
+          mfma32<F16>(sacc[k], A, B);                                                                                     \
         }                                                                                                            \
       }                                                                                                              \
     }                                                                                                                \
@@ -339,7 +339,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
             A[mb].d[1] = lds_read_tr16(p + 4 * VS);                                                                  \
           }                                                                                                          \
           _Pragma("unroll") for (int mb = 0; mb < MB; ++mb)                                                          \
-            _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32(acc[tl][mb][nb], A[mb], B[nb]);                  \
+            _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[tl][mb][nb], A[mb], B[nb]);                  \
         }                                                                                                            \
       }                                                                                                              \
     }                                                                                                                \
@@ -387,7 +387,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) mfma32(acc[tl][mb][nb], A[mb], B[nb]);
+            for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[tl][mb][nb], A[mb], B[nb]);
         }
       }
       // the next tile's first state fragments travel while this one finishes
@@ -458,7 +458,7 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
                 pv[e] = keep ? val : 0.f;
                 rsum += pv[e];
               }
-              *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+              *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack2<F16>(pv[0], pv[1]), pack2<F16>(pv[2], pv[3]));
             }
           }
           if (!IS_DV && own && grp == 0) {
@@ -483,8 +483,8 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
           const uint32_t qq[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
           for (int p = 0; p < 4; ++p) {
-            dot += __uint_as_float(qq[p] << 16) * np[d + 2 * p];
-            dot += __uint_as_float(qq[p] & 0xffff0000u) * np[d + 2 * p + 1];
+            dot += lo2<F16>(qq[p]) * np[d + 2 * p];
+            dot += hi2<F16>(qq[p]) * np[d + 2 * p + 1];
           }
         }
 #pragma unroll
@@ -602,8 +602,8 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
           for (int g4 = 0; g4 < 4; ++g4) {
             const int w0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
             *(uint2*)(Os + (32 * nb + r) * HS + w0) =
-                make_uint2(pack_bf16x2(acc[tl][mb][nb][4 * g4 + 0] * iv + sh, acc[tl][mb][nb][4 * g4 + 1] * iv + sh),
-                           pack_bf16x2(acc[tl][mb][nb][4 * g4 + 2] * iv + sh, acc[tl][mb][nb][4 * g4 + 3] * iv + sh));
+                make_uint2(pack2<F16>(acc[tl][mb][nb][4 * g4 + 0] * iv + sh, acc[tl][mb][nb][4 * g4 + 1] * iv + sh),
+                           pack2<F16>(acc[tl][mb][nb][4 * g4 + 2] * iv + sh, acc[tl][mb][nb][4 * g4 + 3] * iv + sh));
           }
       }
       __syncthreads();
@@ -623,13 +623,13 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
 #undef MLSTM_V_STEP
 }
 
-template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM>
+template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM, bool F16>
 __global__ __launch_bounds__(64 * (WT / MW))
     __attribute__((amdgpu_waves_per_eu(PAR_HV_WPE(WT, MW), PAR_HV_WPE(WT, MW)))) void par_hv_kernel(ParHvArgs a) {
-  par_hv_body<WT, NTG, IS_DV, PD, MW, HEAD_NORM>(a, xcd_block_id());  // the workgroups that share a kept state run on one XCD
+  par_hv_body<WT, NTG, IS_DV, PD, MW, HEAD_NORM, F16>(a, xcd_block_id());  // the workgroups that share a kept state run on one XCD
 }
 
-template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM>
+template <int WT, int NTG, bool IS_DV, int PD, int MW, bool HEAD_NORM, bool F16>
 static const char* launch_par_hv_hn(const ParHvArgs& a, int BH, hipStream_t stream) {
   constexpr int GW = WT * NTG;
   constexpr int VR = 8192 / GW;
@@ -640,20 +640,23 @@ static const char* launch_par_hv_hn(const ParHvArgs& a, int BH, hipStream_t stre
   if (smem > 160 * 1024) return "par_hv: DHQK too large for the LDS-resident tile";
   if ((size_t)a.S * (size_t)(a.DHHV > a.DHQK ? a.DHHV : a.DHQK) * 2 >= ((size_t)1 << 32))
     return "par_hv: one (batch, head) slab of an input exceeds 4 GiB";
-  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, NTG, IS_DV, PD, MW, HEAD_NORM>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)par_hv_kernel<WT, NTG, IS_DV, PD, MW, HEAD_NORM, F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_hv: cannot raise the dynamic LDS limit";
   dim3 grid(2, a.NC, BH);
-  hipLaunchKernelGGL((par_hv_kernel<WT, NTG, IS_DV, PD, MW, HEAD_NORM>), grid, dim3(64 * (WT / MW)), smem, stream, a);
+  hipLaunchKernelGGL((par_hv_kernel<WT, NTG, IS_DV, PD, MW, HEAD_NORM, F16>), grid, dim3(64 * (WT / MW)), smem, stream, a);
   return nullptr;
 }
 
 template <int WT, int NTG, bool IS_DV, int PD, int MW>
 static const char* launch_par_hv_pd(const ParHvArgs& a, int BH, hipStream_t stream) {
   if constexpr (!IS_DV) {
-    if (a.head_norm != 0) return launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, true>(a, BH, stream);
+    if (a.head_norm != 0)
+      return a.f16 ? launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, true, true>(a, BH, stream)
+                   : launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, true, false>(a, BH, stream);
   }
-  return launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, false>(a, BH, stream);
+  return a.f16 ? launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, false, true>(a, BH, stream)
+               : launch_par_hv_hn<WT, NTG, IS_DV, PD, MW, false, false>(a, BH, stream);
 }
 
 template <int WT, int NTG, bool IS_DV>

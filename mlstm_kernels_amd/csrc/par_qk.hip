@@ -37,7 +37,7 @@
 
 namespace mlstm {
 
-template <int MT, bool IS_DQ>
+template <int MT, bool IS_DQ, bool F16>
 __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId blk, const int n_bh) {
   constexpr int NWAVE = MT / 64;    // each wave owns 64 head-dim rows = 2 MFMA row blocks
   constexpr int NTH = 64 * NWAVE;
@@ -173,7 +173,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
       const int obc = ob < 4 ? ob : 3;                                                                               \
       Frag A;                                                                                                        \
       A.u = *(const uint4*)(Xo + (32 * obc + r) * XS + 32 * (sub_) + 16 * ks + 8 * h);                               \
-      _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);                                \
+      _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32<F16>(sacc[k][nb], A, B[nb]);                                \
     }                                                                                                                \
   }
 
@@ -228,7 +228,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
 #pragma unroll
           for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);
+            for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[mb][nb], A[mb], B[nb]);
         }
         // score block: A = Xo rows of the blocks dealt to this wave.  Unconditional on purpose: a wave whose block lies
         // above the diagonal multiplies zero rows (its result is dropped at the gating step); a branch here would make
@@ -240,7 +240,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
           Frag A;
           A.u = *(const uint4*)(Xo + (32 * obc + r) * XS + 32 * sub + 16 * ks + 8 * h);
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) mfma32(sacc[k][nb], A, B[nb]);
+          for (int nb = 0; nb < 2; ++nb) mfma32<F16>(sacc[k][nb], A, B[nb]);
         }
       }
     };
@@ -313,7 +313,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
             const float val = sacc[k][nb][4 * g4 + e] * a.qk_scale * __expf(ex) * rn * ro[e];                        \
             pv[e] = keep ? val : 0.f;                                                                                \
           }                                                                                                          \
-          *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));           \
+          *(uint2*)(Ps + nl * PS + o0) = make_uint2(pack2<F16>(pv[0], pv[1]), pack2<F16>(pv[2], pv[3]));           \
         }                                                                                                            \
       }                                                                                                              \
     }                                                                                                                \
@@ -342,7 +342,7 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
         _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)                                                             \
           B[nb].u = *(const uint4*)(Ps + (32 * nb + r) * PS + 32 * ob + 16 * jl + 8 * h);                            \
         _Pragma("unroll") for (int mb = 0; mb < 2; ++mb)                                                             \
-          _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32(acc[mb][nb], A[mb], B[nb]);                        \
+          _Pragma("unroll") for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[mb][nb], A[mb], B[nb]);                        \
       }                                                                                                              \
     }                                                                                                                \
   }
@@ -444,10 +444,10 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
       for (int g4 = 0; g4 < 4; ++g4) {
         const int d0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
         const uint2 xv = *(const uint2*)(Os + nl * OS + d0);
-        part += acc[mb][nb][4 * g4 + 0] * __uint_as_float(xv.x << 16);
-        part += acc[mb][nb][4 * g4 + 1] * __uint_as_float(xv.x & 0xffff0000u);
-        part += acc[mb][nb][4 * g4 + 2] * __uint_as_float(xv.y << 16);
-        part += acc[mb][nb][4 * g4 + 3] * __uint_as_float(xv.y & 0xffff0000u);
+        part += acc[mb][nb][4 * g4 + 0] * lo2<F16>(xv.x);
+        part += acc[mb][nb][4 * g4 + 1] * hi2<F16>(xv.x);
+        part += acc[mb][nb][4 * g4 + 2] * lo2<F16>(xv.y);
+        part += acc[mb][nb][4 * g4 + 3] * hi2<F16>(xv.y);
       }
     part += __shfl_xor(part, 32);
     if (h == 0) red[wave * 64 + nl] = part;
@@ -470,8 +470,8 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int d0 = m_wave + 32 * mb + 8 * g4 + 4 * h;
-        *(uint2*)(Os + nl * OS + d0) = make_uint2(pack_bf16x2(acc[mb][nb][4 * g4 + 0], acc[mb][nb][4 * g4 + 1]),
-                                                  pack_bf16x2(acc[mb][nb][4 * g4 + 2], acc[mb][nb][4 * g4 + 3]));
+        *(uint2*)(Os + nl * OS + d0) = make_uint2(pack2<F16>(acc[mb][nb][4 * g4 + 0], acc[mb][nb][4 * g4 + 1]),
+                                                  pack2<F16>(acc[mb][nb][4 * g4 + 2], acc[mb][nb][4 * g4 + 3]));
       }
   }
   __syncthreads();
@@ -491,35 +491,40 @@ __device__ __forceinline__ void par_qk_body(const ParQkArgs& a, const BlockId bl
 // dQ and dK of every chunk in ONE launch: the workgroups of a chunk (both gradients, both position halves, all
 // head-dimension tiles) are neighbours in launch order and run on the same XCD at about the same time, so the Q, K, V
 // and dH rows they all stream are fetched from HBM once and served to the others from the caches.
-template <int MT>
+template <int MT, bool F16>
 __global__ __launch_bounds__(MT) __attribute__((amdgpu_waves_per_eu(PAR_QK_WPE(MT), PAR_QK_WPE(MT)))) void par_qk_pair_kernel(ParQkArgs a) {
   BlockId blk = xcd_block_id();
   const int per = 2 * (a.DHQK / MT);
   const int n_bh = (int)gridDim.z;
   if (blk.x < per) {
-    par_qk_body<MT, true>(a, blk, n_bh);
+    par_qk_body<MT, true, F16>(a, blk, n_bh);
   } else {
     blk.x -= per;
     a.states = a.states2;
     a.Out = a.Out2;
     a.rowdot = a.rowdot2;
-    par_qk_body<MT, false>(a, blk, n_bh);
+    par_qk_body<MT, false, F16>(a, blk, n_bh);
   }
 }
 
-template <int MT>
-static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t stream) {
+template <int MT, bool F16>
+static const char* launch_par_qk_pair_f(const ParQkArgs& a, int BH, hipStream_t stream) {
   constexpr int CF = (MT / 16) * 64 * 8;
   constexpr int sa = CF + 64 * 72 + 128 * 72, sb = 64 * (MT + 8), sc = 64 * (MT + 32);
   constexpr int sab = sa > sb ? sa : sb;
   constexpr int stage = sab > sc ? sab : sc;
   const size_t smem = (size_t)(stage + 64 * 136) * 2 + (size_t)(64 * 2 + 128 * 2 + 64 + (MT / 64) * 64) * 4;
-  if (hipFuncSetAttribute((const void*)par_qk_pair_kernel<MT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)par_qk_pair_kernel<MT, F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "par_qk: cannot raise the dynamic LDS limit";
   dim3 grid(4 * (a.DHQK / MT), a.NC, BH);
-  hipLaunchKernelGGL((par_qk_pair_kernel<MT>), grid, dim3(MT), smem, stream, a);
+  hipLaunchKernelGGL((par_qk_pair_kernel<MT, F16>), grid, dim3(MT), smem, stream, a);
   return nullptr;
+}
+
+template <int MT>
+static const char* launch_par_qk_pair_t(const ParQkArgs& a, int BH, hipStream_t stream) {
+  return a.f16 ? launch_par_qk_pair_f<MT, true>(a, BH, stream) : launch_par_qk_pair_f<MT, false>(a, BH, stream);
 }
 
 int par_qk_head_tile(int DHQK) { return DHQK % 256 == 0 ? 256 : (DHQK % 128 == 0 ? 128 : 64); }

@@ -41,7 +41,7 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 #define SCAN_WPE(HILO_, WCOLS_) ((WCOLS_) == 64 && (HILO_) ? 1 : 2)
 // WCOLS = value columns per wave (64 or 32): with 32 a 128 x 128 tile takes eight waves, two per SIMD, each with
 // half the staging work and half the accumulators.
-template <int RT, int WT, bool HILO, int PS, int WCOLS>
+template <int RT, int WT, bool HILO, int PS, int WCOLS, bool F16>
 __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     __attribute__((amdgpu_waves_per_eu(SCAN_WPE(HILO, WCOLS), SCAN_WPE(HILO, WCOLS)))) void scan_kernel(ScanArgs a) {
   constexpr int WC = WT / WCOLS;
@@ -188,8 +188,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
         const float xsc = scur[j];
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-          np[2 * p] += xsc * __uint_as_float(in[p] << 16);
-          np[2 * p + 1] += xsc * __uint_as_float(in[p] & 0xffff0000u);
+          np[2 * p] += xsc * lo2<F16>(in[p]);
+          np[2 * p + 1] += xsc * hi2<F16>(in[p]);
         }
       }
     }
@@ -208,10 +208,10 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       const float sc = scur[j];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const float e0 = __uint_as_float(in[p] << 16) * sc;
-        const float e1 = __uint_as_float(in[p] & 0xffff0000u) * sc;
-        hi[p] = pack_bf16x2(e0, e1);
-        if (HILO) lo[p] = pack_bf16x2(e0 - __uint_as_float(hi[p] << 16), e1 - __uint_as_float(hi[p] & 0xffff0000u));
+        const float e0 = lo2<F16>(in[p]) * sc;
+        const float e1 = hi2<F16>(in[p]) * sc;
+        hi[p] = pack2<F16>(e0, e1);
+        if (HILO) lo[p] = pack2<F16>(e0 - lo2<F16>(hi[p]), e1 - hi2<F16>(hi[p]));
       }
       *(uint4*)(Yh + j * YS + cv * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
       if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
@@ -236,10 +236,10 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             uint4 f;
-            f.x = pack_bf16x2(acc[db][wb][8 * half + 0], acc[db][wb][8 * half + 1]);
-            f.y = pack_bf16x2(acc[db][wb][8 * half + 2], acc[db][wb][8 * half + 3]);
-            f.z = pack_bf16x2(acc[db][wb][8 * half + 4], acc[db][wb][8 * half + 5]);
-            f.w = pack_bf16x2(acc[db][wb][8 * half + 6], acc[db][wb][8 * half + 7]);
+            f.x = pack2<F16>(acc[db][wb][8 * half + 0], acc[db][wb][8 * half + 1]);
+            f.y = pack2<F16>(acc[db][wb][8 * half + 2], acc[db][wb][8 * half + 3]);
+            f.z = pack2<F16>(acc[db][wb][8 * half + 4], acc[db][wb][8 * half + 5]);
+            f.w = pack2<F16>(acc[db][wb][8 * half + 6], acc[db][wb][8 * half + 7]);
             // non-temporal: the fragments are read by a later kernel; kept out of the L2 they do not evict the K/V
             // rows the tiles of a head share
             const u32x4 fv = {f.x, f.y, f.z, f.w};
@@ -281,8 +281,8 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       for (int db = 0; db < 2; ++db)
 #pragma unroll
         for (int wb = 0; wb < NBW; ++wb) {
-          mfma32(acc[db][wb], A[db], Bh[wb]);
-          if (HILO) mfma32(acc[db][wb], A[db], Bl[wb]);
+          mfma32<F16>(acc[db][wb], A[db], Bh[wb]);
+          if (HILO) mfma32<F16>(acc[db][wb], A[db], Bl[wb]);
         }
     }
     // ---- normaliser vector (forward, first column tile only): n = gbar n + sum_j abar_j k_j
@@ -310,20 +310,25 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   if (do_n && tid < RT && a.n_final != nullptr) a.n_final[(size_t)bh * DHQK + d_tile + tid] = nval;
 }
 
-template <int RT, int WT, bool HILO>
-static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
+template <int RT, int WT, bool HILO, bool F16>
+static const char* launch_scan_f(const ScanArgs& a, int BH, hipStream_t stream) {
   constexpr int WCOLS = 32;
   constexpr int NT = 64 * (RT / 64) * (WT / WCOLS);
   constexpr int XROWS = NT / (RT / 8);
   constexpr int PS = 128;
   const size_t smem = (size_t)PS * (RT + 32) * 2 + (size_t)PS * (WT + 32) * 2 * (HILO ? 2 : 1) +
                       (size_t)(XROWS * RT + kGBlock + 2 * kChunk) * 4;
-  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS, WCOLS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+  if (hipFuncSetAttribute((const void*)scan_kernel<RT, WT, HILO, PS, WCOLS, F16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)smem) != hipSuccess)
     return "scan: cannot raise the dynamic LDS limit";
   dim3 grid(a.DHQK / RT, a.DHHV / WT, BH);
-  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO, PS, WCOLS>), grid, dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL((scan_kernel<RT, WT, HILO, PS, WCOLS, F16>), grid, dim3(NT), smem, stream, a);
   return nullptr;
+}
+
+template <int RT, int WT, bool HILO>
+static const char* launch_scan_t(const ScanArgs& a, int BH, hipStream_t stream) {
+  return a.f16 ? launch_scan_f<RT, WT, HILO, true>(a, BH, stream) : launch_scan_f<RT, WT, HILO, false>(a, BH, stream);
 }
 
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream) {

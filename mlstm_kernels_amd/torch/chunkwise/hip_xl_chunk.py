@@ -10,9 +10,10 @@ because the chunkwise formulation is exact for every chunk length.  ``chunk_size
 1024) selects how far apart the kept chunk states are, as in the reference (``save_states_every_nth_chunk`` =
 ``chunk_size_intra // chunk_size_inter``); the Triton tile-size and launch keywords are accepted and ignored.
 
-Arithmetic: the matrix cores multiply bf16 operands and accumulate in fp32; gates, stabilisers, normalisers and
-states are fp32.  float32 and float16 inputs (or ``autocast_kernel_dtype``) are therefore rounded to bfloat16 at the
-boundary -- unlike the reference's Triton kernels, which run in the requested dtype -- and a warning says so once."""
+Arithmetic: the matrix cores multiply bfloat16 or float16 operands -- the dtype of q after the autocast cast to
+``autocast_kernel_dtype`` -- and accumulate in fp32; gates, stabilisers, normalisers and states are fp32.  float32
+inputs are rounded to bfloat16 at the boundary -- unlike the reference's Triton kernels, which then multiply in
+tf32 -- and a warning says so once."""
 from __future__ import annotations
 
 import warnings
@@ -35,10 +36,9 @@ def _warn_rounding_once(dtype: torch.dtype) -> None:
     if dtype not in _warned_rounding:
         _warned_rounding.add(dtype)
         warnings.warn(
-            f"mlstm_kernels_amd: {dtype} operands are rounded to bfloat16 for the HIP chunkwise kernels (bf16 matrix "
+            f"mlstm_kernels_amd: {dtype} operands are rounded to bfloat16 for the HIP chunkwise kernels (16-bit matrix "
             "cores with fp32 accumulation; gates, normalisers and states stay fp32). "
-            + ("float16 loses three mantissa bits this way. " if dtype == torch.float16 else "")
-            + "Pass bfloat16 tensors and autocast_kernel_dtype=torch.bfloat16 to make this explicit.",
+            "Pass bfloat16 or float16 tensors to choose the operand format yourself.",
             stacklevel=4,
         )
 
@@ -81,6 +81,8 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
     DHHV = v.shape[-1]
     dev = q.device
     lib = _lib.get_lib()
+    if path == _lib.PATH_FUSED and q.dtype != torch.bfloat16:
+        raise RuntimeError(f"the fused kernel path supports bfloat16 operands only, got {q.dtype}")
     ws_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, int(keep), path, stride)
     if ws_bytes == 0:
         if DHQK % 64 == 0 and DHQK > 896:
@@ -92,7 +94,7 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
             "(head dimensions must be multiples of 64, DHQK <= 896, B*NH <= 65535)"
         )
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
+    H = torch.empty(B, NH, S, DHHV, dtype=q.dtype, device=dev)
     if norm != _lib.NORM_NONE:
         if DHHV not in (64, 128, 256, 512):
             raise ValueError(f"the fused head norm needs DHHV = 64, 128, 256 or 512, got {DHHV}")
@@ -110,7 +112,7 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
         ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0),
         ptr(H), None, None, ptr(c_last), ptr(n_last), ptr(m_last),
         ptr(ws), ws_bytes, int(keep), B, NH, S, DHQK, DHHV, float(eps),
-        _lib.BF16, dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
+        dtype_code(q), dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
         norm, float(norm_eps), ptr(norm_mean), ptr(norm_rstd), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_chunkwise_fw")
@@ -123,12 +125,13 @@ def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
     assert k.shape == (B, NH, S, DHQK), f"k has wrong shape {tuple(k.shape)}"
     assert v.shape[:3] == (B, NH, S), f"v has wrong shape {tuple(v.shape)}"
     assert i.shape == (B, NH, S) and f.shape == (B, NH, S), "i and f must have shape (B, NH, S)"
-    bf = torch.bfloat16
+    # operand format of the matrix kernels: float16 when q is float16, bfloat16 otherwise
+    kd = torch.float16 if q.dtype == torch.float16 else torch.bfloat16
     for t in (q, k, v):
-        if t.dtype != bf:
+        if t.dtype == torch.float32:
             _warn_rounding_once(t.dtype)
-    qb, kb, vb = (t.to(bf).contiguous() for t in (q, k, v))
-    gate_dt = torch.bfloat16 if (i.dtype == bf and f.dtype == bf) else torch.float32
+    qb, kb, vb = (t.to(kd).contiguous() for t in (q, k, v))
+    gate_dt = i.dtype if (i.dtype == f.dtype and i.dtype in (torch.bfloat16, torch.float16)) else torch.float32
     ib, fb = i.to(gate_dt).contiguous(), f.to(gate_dt).contiguous()
     if c0 is not None:
         assert n0 is not None, "Initial states must be provided together."
@@ -163,7 +166,7 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
                 ctx.save_for_backward(qb, kb, vb, ib, fb, ws)
             ctx.cfg = (eps, q.dtype, k.dtype, v.dtype, i.dtype, f.dtype,
                        None if c0 is None else c0.dtype, n0 is not None, m0 is not None)
-            H = H if out_dtype == torch.bfloat16 else H.to(out_dtype)
+            H = H if out_dtype == H.dtype else H.to(out_dtype)
             return H, c_last, n_last, m_last
 
         @staticmethod
@@ -178,14 +181,14 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
             bw_bytes = lib.mlstm_hip_chunkwise_bw_workspace_bytes(B, NH, S, DHQK, DHHV, stride)
             bws = torch.empty(bw_bytes, dtype=torch.uint8, device=dev)
             if dH is None:  # only the last states are differentiated
-                dH = torch.zeros(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
-            dHb = dH.to(torch.bfloat16).contiguous()
+                dH = torch.zeros(B, NH, S, DHHV, dtype=qb.dtype, device=dev)
+            dHb = dH.to(qb.dtype).contiguous()
             if normed:
                 # gradient of the normalised rows -> gradient of H (the un-normalised rows were never stored)
                 Hn, rstd = normed
                 dHraw = torch.empty_like(dHb)
                 rc = lib.mlstm_hip_head_norm_bw(ptr(dHb), ptr(Hn), ptr(rstd), ptr(dHraw), B * NH * S, DHHV, norm,
-                                                _lib.BF16, current_stream_ptr(dev))
+                                                dtype_code(dHb), current_stream_ptr(dev))
                 _lib.check(rc, "mlstm_hip_head_norm_bw")
                 dHb = dHraw
             dCl = None if dC_last is None else dC_last.to(torch.float32).contiguous()
@@ -197,7 +200,7 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
                 ptr(qb), ptr(kb), ptr(vb), ptr(ib), ptr(fb), ptr(dHb), ptr(dCl),
                 ptr(dQ), ptr(dK), ptr(dV), ptr(dI), ptr(dF), ptr(dC0),
                 ptr(ws), ws.numel(), ptr(bws), bw_bytes, B, NH, S, DHQK, DHHV, float(eps),
-                _lib.BF16, dtype_code(ib), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
+                dtype_code(qb), dtype_code(ib), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
                 current_stream_ptr(dev),
             )
             _lib.check(rc, "mlstm_hip_chunkwise_bw")
@@ -247,8 +250,8 @@ def mlstm_chunkwise__hip_xl_chunk(
 ):
     """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
     ``(H, (C_last fp32 (B,NH,DHQK,DHHV), n_last fp32 (B,NH,DHQK), m_last fp32 (B,NH,1)))``.
-    The matrix kernels multiply in bf16 with fp32 accumulation whatever the input dtype (other dtypes are rounded to
-    bf16, with a one-time warning).
+    The matrix kernels multiply in the dtype of q -- bfloat16 or float16 -- with fp32 accumulation; float32 inputs
+    are rounded to bfloat16, with a one-time warning.
     ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
     tail themselves, so every S >= 1 is one call.  ``kernel_path`` ("auto", "split", "fused"; not in the reference)
     selects the kernels of the value-column side.  ``chunk_size_intra`` (reference keyword) sets the distance between

@@ -11,13 +11,13 @@ def dtype_code(t: torch.Tensor) -> int:
         return _lib.F32
     if t.dtype == torch.bfloat16:
         return _lib.BF16
-    raise TypeError(f"unsupported dtype {t.dtype}: the HIP kernels take float32 or bfloat16 tensors")
+    if t.dtype == torch.float16:
+        return _lib.F16
+    raise TypeError(f"unsupported dtype {t.dtype}: the HIP kernels take float32, bfloat16 or float16 tensors")
 
 
 def state_dtype_code(t: torch.Tensor) -> int:
     """dtype code of a recurrent state tensor (float32, bfloat16 or float16)."""
-    if t.dtype == torch.float16:
-        return _lib.F16
     return dtype_code(t)
 
 
