@@ -8,7 +8,8 @@ with the same argument names, defaults, return structure and shape rules
 internal chunks of 128 positions (the reference's ``chunk_size_inter``), which leaves H and the last states unchanged
 because the chunkwise formulation is exact for every chunk length.  ``chunk_size_intra`` (a multiple of 128, at most
 1024) selects how far apart the kept chunk states are, as in the reference (``save_states_every_nth_chunk`` =
-``chunk_size_intra // chunk_size_inter``); the Triton tile-size and launch keywords are accepted and ignored.
+``chunk_size_intra // chunk_size_inter``); ``chunk_size_inter`` is checked and otherwise has no effect; the Triton
+tile-size and launch keywords are accepted and ignored.
 
 Arithmetic: the matrix cores multiply bfloat16 or float16 operands -- the dtype of q after the autocast cast to
 ``autocast_kernel_dtype`` -- and accumulate in fp32; gates, stabilisers, normalisers and states are fp32.  float32
@@ -44,19 +45,28 @@ def _warn_rounding_once(dtype: torch.dtype) -> None:
 
 
 def _state_stride(tuning_kwargs: dict, who: str) -> int:
-    """chunk_size_inter / chunk_size_intra of the reference (kernel_param_heuristics.py:118-121) -> state stride."""
+    """chunk_size_inter / chunk_size_intra of the reference (kernel_param_heuristics.py:118-121) -> state stride.
+
+    The reference scans in chunks of chunk_size_inter and keeps a state every chunk_size_intra positions.  The HIP
+    scan always runs in chunks of 128 positions -- the results do not depend on the chunk of the scan -- so
+    chunk_size_inter only has to be a value the reference would take (a power of two from 16 to 128 that divides
+    chunk_size_intra); chunk_size_intra sets the distance between kept states, in units of 128 positions (a smaller
+    value keeps a state per internal chunk)."""
     for key in tuning_kwargs:
         if key not in _IGNORED_TUNING_KWARGS and key not in ("chunk_size_inter", "chunk_size_intra"):
             raise TypeError(f"{who}() got an unexpected keyword argument '{key}'")
     inter = tuning_kwargs.get("chunk_size_inter")
     intra = tuning_kwargs.get("chunk_size_intra")
-    if inter is not None and inter != _INTERNAL_CHUNK:
-        raise ValueError(f"the HIP kernels scan in chunks of {_INTERNAL_CHUNK} positions: chunk_size_inter must be "
-                         f"{_INTERNAL_CHUNK} or None, got {inter}")
+    if inter is not None and inter not in (16, 32, 64, _INTERNAL_CHUNK):
+        raise ValueError(f"chunk_size_inter must be 16, 32, 64 or {_INTERNAL_CHUNK} (or None), got {inter}")
     if intra is None:
         return 0
-    if intra % _INTERNAL_CHUNK != 0 or not (1 <= intra // _INTERNAL_CHUNK <= 8):
-        raise ValueError(f"chunk_size_intra must be a multiple of {_INTERNAL_CHUNK} between {_INTERNAL_CHUNK} and "
+    if inter is not None and (intra < inter or intra % inter != 0):
+        raise ValueError(f"chunk_size_intra ({intra}) must be a multiple of chunk_size_inter ({inter})")
+    if intra in (16, 32, 64):
+        return 1
+    if intra <= 0 or intra % _INTERNAL_CHUNK != 0 or intra // _INTERNAL_CHUNK > 8:
+        raise ValueError(f"chunk_size_intra must be 16, 32, 64 or a multiple of {_INTERNAL_CHUNK} up to "
                          f"{8 * _INTERNAL_CHUNK}, got {intra}")
     return intra // _INTERNAL_CHUNK
 

@@ -87,7 +87,10 @@ def test_operator_options_are_validated_on_the_host():
     assert _state_stride({"chunk_size_intra": 128}, "op") == 1
     assert _state_stride({"chunk_size_inter": 128, "chunk_size_intra": 512}, "op") == 4
     assert _state_stride({"siz_b_L_parallel": 64, "num_warps_intra": 4, "recompute_states_in_bw": True}, "op") == 0
-    for bad in ({"chunk_size_inter": 64}, {"chunk_size_intra": 192}, {"chunk_size_intra": 2048}, {"chunk_size_intra": 0}):
+    assert _state_stride({"chunk_size_inter": 64, "chunk_size_intra": 256}, "op") == 2   # the scan's own chunk stays 128
+    assert _state_stride({"chunk_size_inter": 64, "chunk_size_intra": 64}, "op") == 1
+    for bad in ({"chunk_size_inter": 96}, {"chunk_size_inter": 256}, {"chunk_size_intra": 192}, {"chunk_size_intra": 2048},
+                {"chunk_size_intra": 0}, {"chunk_size_inter": 128, "chunk_size_intra": 64}):
         with pytest.raises(ValueError):
             _state_stride(bad, "op")
     with pytest.raises(TypeError, match="unexpected keyword"):
