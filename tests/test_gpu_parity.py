@@ -532,6 +532,31 @@ def test_chunkwise_fwbw_xlstm7b_shape_sig():
     _fwbw_case(4, 8, 16384, 256, 512, siging=True, init=True, seed=0, pairs=[(1, 4), (2, 3)])   # middle of the grid
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("siging", [False, True])
+def test_chunkwise_takes_16_bit_gates(dtype, siging):
+    """Gate pre-activations in the operand dtype (what a model under autocast hands over): the kernels read them in
+    that format; the oracle gets the same rounded values.  dI/dF come back in the gate dtype."""
+    exp_op, sig_op, *_ = _ops()
+    B, NH, S, DQK, DHV = 2, 2, 384, 128, 256
+    q, k, v, i, f = make_qkvif(B, NH, S, DQK, DHV, seed=21, dtype=dtype)
+    i, f = i.to(dtype), f.to(dtype)
+    g = torch.Generator().manual_seed(4)
+    dH = torch.randn(B, NH, S, DHV, generator=g).to(dtype)
+    fw = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=128, siging=siging, return_bounds=True)
+    bw = O.chunkwise_bw(*(d64(t) for t in (q, k, v, i, f)), d64(dH), chunk_size=128, siging=siging)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (q, k, v, i, f)]
+    H = (sig_op if siging else exp_op)(*leaves, chunk_size=128)
+    H.backward(dH.to(DEV))
+    unit = _U_F16 if dtype == torch.float16 else _U_BF16
+    check_matrix(H, fw["H"], "H", abs_sum=fw["H_abs"], unit=unit)
+    for name, leaf, r in zip(["dQ", "dK", "dV"], leaves[:3], bw[:3]):
+        check_matrix(leaf.grad, r, name)
+    for name, leaf, r in zip(["dI", "dF"], leaves[3:], bw[3:5]):
+        assert leaf.grad.dtype == dtype
+        assert rel_to_scale(leaf.grad, r) <= 5e-2, name
+
+
 # ------------------------------------------------------------------------------------------ size-independent properties
 def test_state_passing_and_exact_value_scaling_at_full_size():
     exp_op, *_ = _ops()
