@@ -13,7 +13,7 @@
  *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1, MLSTM_F16 = 2.  The chunkwise entry points take q/k/v (and dH) in
  *     bf16 or fp16 and multiply in that format on the matrix cores with fp32 accumulation (the kept chunk states are
  *     rounded to the same format; fp16 has three more mantissa bits and overflows above 65504); gates in fp32, bf16 or
- *     fp16.  The decode entry points take q/k/v and gates in fp32 or bf16 and states in fp32, bf16 or fp16.
+ *     fp16.  The decode entry points take q/k/v, gates and states in fp32, bf16 or fp16 each (fp32 arithmetic).
  *   - gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp), MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
  *   - Supported shapes: DHQK % 64 == 0 (at most 896), DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
  *

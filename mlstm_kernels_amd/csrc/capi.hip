@@ -90,6 +90,8 @@ namespace mlstm {
 int set_last_error(const char* msg) { return fail(msg); }
 }  // namespace mlstm
 
+static bool valid_dtype(int code) { return code == MLSTM_F32 || code == MLSTM_BF16 || code == MLSTM_F16; }
+
 extern "C" {
 
 int mlstm_hip_abi_version(void) { return 5; }
@@ -139,8 +141,7 @@ int mlstm_hip_step(const void* q, const void* k, const void* v, const void* i, c
     return fail("mlstm_hip_step: null pointer argument");
   if (n_out == n_in || m_out == m_in)
     return fail("mlstm_hip_step: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
-  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) ||
-      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16 && dtype_state != MLSTM_F16))
+  if (!valid_dtype(dtype_qkv) || !valid_dtype(dtype_gates) || !valid_dtype(dtype_state))
     return fail("mlstm_hip_step: unsupported dtype code");
   {
     ProfileScope ps("step", (hipStream_t)stream);
@@ -159,8 +160,7 @@ int mlstm_hip_recurrent_sequence(const void* q, const void* k, const void* v, co
     return fail("mlstm_hip_recurrent_sequence: null pointer argument");
   if (n_out == n_in || m_out == m_in)
     return fail("mlstm_hip_recurrent_sequence: n_out/m_out must not alias n_in/m_in (only C may be updated in place)");
-  if ((dtype_qkv != MLSTM_F32 && dtype_qkv != MLSTM_BF16) || (dtype_gates != MLSTM_F32 && dtype_gates != MLSTM_BF16) ||
-      (dtype_state != MLSTM_F32 && dtype_state != MLSTM_BF16 && dtype_state != MLSTM_F16))
+  if (!valid_dtype(dtype_qkv) || !valid_dtype(dtype_gates) || !valid_dtype(dtype_state))
     return fail("mlstm_hip_recurrent_sequence: unsupported dtype code");
   {
     ProfileScope ps("step_seq", (hipStream_t)stream);

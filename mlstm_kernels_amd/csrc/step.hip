@@ -144,10 +144,8 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
 #pragma unroll
       for (int e4 = 0; e4 < VPL / 4; ++e4) {
         const uint2 raw = *(const uint2*)((const uint16_t*)v + o + 4 * e4);
-        vv[4 * e4 + 0] = __uint_as_float(raw.x << 16);
-        vv[4 * e4 + 1] = __uint_as_float(raw.x & 0xffff0000u);
-        vv[4 * e4 + 2] = __uint_as_float(raw.y << 16);
-        vv[4 * e4 + 3] = __uint_as_float(raw.y & 0xffff0000u);
+        unpack_state2(raw.x, dtype_qkv, vv[4 * e4 + 0], vv[4 * e4 + 1]);   // dtype code 1 bf16, 2 fp16
+        unpack_state2(raw.y, dtype_qkv, vv[4 * e4 + 2], vv[4 * e4 + 3]);
       }
     }
   }
@@ -200,8 +198,7 @@ __global__ __launch_bounds__((COLS / StatePiece<SBF>::N) * TY) void step_kernel(
       for (int y = 0; y < TY; ++y) s += red[y * COLS + cidx];
       s *= inv_den;
       const size_t o = (size_t)bh * DHHV + col0 + cidx;
-      if (dtype_qkv == 0) ((float*)h)[o] = s;
-      else ((uint16_t*)h)[o] = f32_to_bf16_bits(s);
+      store_state_scalar(h, o, dtype_qkv, s);   // fp32, bf16 or fp16
     }
   }
 }

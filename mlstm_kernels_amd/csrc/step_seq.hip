@@ -43,7 +43,7 @@ constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i inside each row of 1
 
 // waves per SIMD the register budget is cut for: the state slice takes RPT * CPT registers per lane
 #define STEP_SEQ_WPE(REGS_) ((REGS_) <= 64 ? 3 : 2)
-template <int RPT, int CPT, bool VEC, bool BF16>
+template <int RPT, int CPT, bool VEC, int QDT>
 __global__ __launch_bounds__(64)
     __attribute__((amdgpu_waves_per_eu(STEP_SEQ_WPE(RPT * CPT), STEP_SEQ_WPE(RPT * CPT)))) void step_seq_kernel(
     const void* __restrict__ q, const void* __restrict__ k, const void* __restrict__ v,
@@ -121,6 +121,8 @@ __global__ __launch_bounds__(64)
   // Addresses are a uniform base (scalar registers, advanced per token by the scalar unit) plus a constant 32-bit
   // byte offset per lane.
   float qv[PF][NDJ], kv[PF][NDJ], vv[PF][CPT];
+  constexpr bool BF16 = QDT != 0;      // q/k/v and h are 16-bit values: bfloat16 (QDT 1) or float16 (QDT 2)
+  constexpr bool QF16 = QDT == 2;
   constexpr uint32_t ESZ = BF16 ? 2 : 4;
   uint32_t qoff[NDJ], voff[CPT];
 #pragma unroll
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(64)
   const char* const k_bh = (const char*)k + (size_t)bh * T * DHQK * ESZ;
   const char* const v_bh = (const char*)v + (size_t)bh * T * DHHV * ESZ;
   auto ld = [&](const char* base, uint32_t off) -> float {
-    if constexpr (BF16) return __uint_as_float((uint32_t)(*(const uint16_t*)(base + off)) << 16);
+    if constexpr (BF16) return elem_to_f32<QF16>(*(const uint16_t*)(base + off));
     else return *(const float*)(base + off);
   };
   auto fetch = [&](int t_, float (&qd)[NDJ], float (&kd)[NDJ], float (&vc)[CPT]) {
@@ -148,10 +150,10 @@ __global__ __launch_bounds__(64)
       // four neighbouring columns in one piece (past the last column: the piece at column 0, zeroed below)
       if constexpr (BF16) {
         const uint2 raw = *(const uint2*)(vt + (col_in ? voff[0] : 0u));
-        vc[0] = __uint_as_float(raw.x << 16);
-        vc[1 % CPT] = __uint_as_float(raw.x & 0xffff0000u);
-        vc[2 % CPT] = __uint_as_float(raw.y << 16);
-        vc[3 % CPT] = __uint_as_float(raw.y & 0xffff0000u);
+        vc[0] = lo2<QF16>(raw.x);
+        vc[1 % CPT] = hi2<QF16>(raw.x);
+        vc[2 % CPT] = lo2<QF16>(raw.y);
+        vc[3 % CPT] = hi2<QF16>(raw.y);
       } else {
         const f32x4 raw = *(const f32x4*)(vt + (col_in ? voff[0] : 0u));
 #pragma unroll
@@ -289,8 +291,8 @@ __global__ __launch_bounds__(64)
               const f32x4 y = {acc[0] * inv_den, acc[1 % CPT] * inv_den, acc[2 % CPT] * inv_den, acc[3 % CPT] * inv_den};
               *(f32x4*)((float*)h + o) = y;
             } else {
-              *(uint2*)((uint16_t*)h + o) = make_uint2(pack_bf16x2(acc[0] * inv_den, acc[1 % CPT] * inv_den),
-                                                       pack_bf16x2(acc[2 % CPT] * inv_den, acc[3 % CPT] * inv_den));
+              *(uint2*)((uint16_t*)h + o) = make_uint2(pack2<QF16>(acc[0] * inv_den, acc[1 % CPT] * inv_den),
+                                                       pack2<QF16>(acc[2 % CPT] * inv_den, acc[3 % CPT] * inv_den));
             }
           }
         } else {
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(64)
             if (col + e < DHHV) {
               const float s = acc[e] * inv_den;
               if constexpr (!BF16) ((float*)h)[o + e] = s;
-              else ((uint16_t*)h)[o + e] = f32_to_bf16_bits(s);
+              else ((uint16_t*)h)[o + e] = f32_to_elem<QF16>(s);
             }
         }
       }
@@ -339,14 +341,14 @@ __global__ __launch_bounds__(64)
   }
 }
 
-template <int RPT, int CPT, bool VEC, bool BF16>
+template <int RPT, int CPT, bool VEC, int QDT>
 static const char* launch_step_seq_t(const void* q, const void* k, const void* v, const void* i, const void* f,
                                      const void* c_in, const void* n_in, const void* m_in, void* h, void* c_out,
                                      void* n_out, void* m_out, int B, int NH, int T, int DHQK, int DHHV, float eps,
                                      int dtype_qkv, int dtype_gates, int dtype_state, hipStream_t stream) {
   constexpr int COLS = 8 * CPT;
   dim3 grid((DHHV + COLS - 1) / COLS, B * NH);
-  hipLaunchKernelGGL((step_seq_kernel<RPT, CPT, VEC, BF16>), grid, dim3(64), 0, stream, q, k, v, i, f, c_in, n_in, m_in, h,
+  hipLaunchKernelGGL((step_seq_kernel<RPT, CPT, VEC, QDT>), grid, dim3(64), 0, stream, q, k, v, i, f, c_in, n_in, m_in, h,
                      c_out, n_out, m_out, T, DHQK, DHHV, eps, dtype_gates, dtype_state);
   return nullptr;
 }
@@ -360,9 +362,11 @@ const char* launch_step_seq(const void* q, const void* k, const void* v, const v
   if (DHQK > 1024) return "mlstm_hip_recurrent_sequence: DHQK above 1024 does not fit the register-resident state slice";
 #define MLSTM_SEQ_ARGS q, k, v, i, f, c_in, n_in, m_in, h, c_out, n_out, m_out, B, NH, T, DHQK, DHHV, eps, dtype_qkv, dtype_gates, dtype_state, stream
   // rows per lane x columns per lane: at most 128 state registers per lane
-  const bool vec = DHHV % 4 == 0, bf = dtype_qkv != 0;
-#define MLSTM_SEQ_PICK(RPT_, CPT_, VEC_) \
-  return bf ? launch_step_seq_t<RPT_, CPT_, VEC_, true>(MLSTM_SEQ_ARGS) : launch_step_seq_t<RPT_, CPT_, VEC_, false>(MLSTM_SEQ_ARGS)
+  const bool vec = DHHV % 4 == 0;
+#define MLSTM_SEQ_PICK(RPT_, CPT_, VEC_)                                                          \
+  return dtype_qkv == 0   ? launch_step_seq_t<RPT_, CPT_, VEC_, 0>(MLSTM_SEQ_ARGS)                \
+         : dtype_qkv == 1 ? launch_step_seq_t<RPT_, CPT_, VEC_, 1>(MLSTM_SEQ_ARGS)                \
+                          : launch_step_seq_t<RPT_, CPT_, VEC_, 2>(MLSTM_SEQ_ARGS)
   if (DHQK <= 128) {
     if (vec) MLSTM_SEQ_PICK(16, 4, true);
     MLSTM_SEQ_PICK(16, 4, false);

@@ -19,12 +19,6 @@ def _check_state_dtype(dtype_state: torch.dtype) -> torch.dtype:
     return dtype_state
 
 
-def _decode_dtype(t: torch.Tensor) -> torch.dtype:
-    """The decode kernels read q/k/v and the gates as float32 or bfloat16 (their arithmetic is float32 anyway);
-    float16 tensors are widened to float32, which is exact."""
-    return torch.float32 if t.dtype == torch.float16 else t.dtype
-
-
 def mlstm_recurrent_step__hip_fw(
     matC_old: torch.Tensor,  # (B, NH, DHQK, DHHV)
     vecN_old: torch.Tensor,  # (B, NH, DHQK)
@@ -56,8 +50,8 @@ def mlstm_recurrent_step__hip_fw(
         raise NotImplementedError("the HIP step kernel uses qk_scale = DHQK**-0.5")
     dtype_state = _check_state_dtype(dtype_state)
     dev = require_gpu(vecQ, vecK, vecV, scaI, scaF, matC_old, vecN_old, scaM_old)
-    qdt, gdt = _decode_dtype(vecQ), _decode_dtype(scaI)
-    q, k, v = vecQ.to(qdt).contiguous(), vecK.to(qdt).contiguous(), vecV.to(qdt).contiguous()
+    qdt, gdt = vecQ.dtype, scaI.dtype   # float32, bfloat16 or float16 each; the arithmetic is float32
+    q, k, v = vecQ.contiguous(), vecK.to(qdt).contiguous(), vecV.to(qdt).contiguous()
     i, f = scaI.to(gdt).contiguous(), scaF.to(gdt).contiguous()
     c_old = matC_old.to(dtype_state).contiguous()
     n_old = vecN_old.to(dtype_state).contiguous()
@@ -79,7 +73,7 @@ def mlstm_recurrent_step__hip_fw(
         B, NH, DHQK, DHHV, float(eps), dtype_code(q), dtype_code(i), state_dtype_code(c_old), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_step")
-    return h.to(vecQ.dtype), (matC_new, vecN_new, scaM_new)
+    return h, (matC_new, vecN_new, scaM_new)
 
 
 def mlstm_recurrent_step__hip(
@@ -141,8 +135,8 @@ def mlstm_recurrent_sequence__hip(
     if S == 0:
         H = torch.empty(B, NH, 0, DHHV, dtype=q.dtype, device=dev)
         return (H, (c.clone(), n.clone(), m.clone())) if return_last_states else H
-    qdt, gdt = _decode_dtype(q), _decode_dtype(i)
-    qc, kc, vc = q.to(qdt).contiguous(), k.to(qdt).contiguous(), v.to(qdt).contiguous()
+    qdt, gdt = q.dtype, i.dtype
+    qc, kc, vc = q.contiguous(), k.to(qdt).contiguous(), v.to(qdt).contiguous()
     ic, fc = i.to(gdt).contiguous(), f.to(gdt).contiguous()
     H = torch.empty(B, NH, S, DHHV, dtype=qdt, device=dev)
     c_out, n_out, m_out = torch.empty_like(c), torch.empty_like(n), torch.empty_like(m)
@@ -153,7 +147,6 @@ def mlstm_recurrent_sequence__hip(
         B, NH, S, DHQK, DHHV, float(eps), dtype_code(qc), dtype_code(ic), state_dtype_code(c), current_stream_ptr(dev),
     )
     _lib.check(rc, "mlstm_hip_recurrent_sequence")
-    H = H.to(q.dtype)
     if return_last_states:
         return H, (c_out, n_out, m_out)
     return H

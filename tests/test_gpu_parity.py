@@ -153,7 +153,7 @@ def test_step_parity(B, NH, DQK, DHV, dtype):
 
 @pytest.mark.parametrize("B,NH,DQK,DHV", [(2, 2, 64, 128), (3, 4, 256, 512), (3, 2, 96, 100)])
 def test_step_and_sequence_take_float16_inputs(B, NH, DQK, DHV):
-    """float16 q/k/v and gates: the decode wrappers widen them to float32 (exact), h comes back in float16."""
+    """float16 q/k/v and gates are read by the decode kernels as they are (fp32 arithmetic), h comes back in float16."""
     *_, step, seq = _ops()
     g = torch.Generator().manual_seed(17)
     T = 5
