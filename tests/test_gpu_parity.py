@@ -557,6 +557,53 @@ def test_chunkwise_takes_16_bit_gates(dtype, siging):
         assert rel_to_scale(leaf.grad, r) <= 5e-2, name
 
 
+def test_chunkwise_fwbw_in_hip_graph():
+    """Forward and backward of the chunkwise operator captured once in a HIP graph (workspaces from the graph's memory
+    pool, no memset nodes: the library clears with fill kernels) and replayed on new data, with eager passes between
+    the replays: every replay must reproduce the eager result bit for bit."""
+    exp_op, *_ = _ops()
+    B, NH, S, DQK, DHV = 2, 4, 1024, 256, 512
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gen)
+    data = [[rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DQK).bfloat16(), rn(B, NH, S, DHV).bfloat16(), rn(B, NH, S),
+             3 + rn(B, NH, S), rn(B, NH, S, DHV).bfloat16()] for _ in range(3)]
+
+    def eager(d):
+        leaves = [t.clone().requires_grad_(True) for t in d[:5]]
+        H = exp_op(*leaves, chunk_size=128)
+        H.backward(d[5])
+        return [H.detach().clone()] + [t.grad.clone() for t in leaves]
+
+    refs = [eager(d) for d in data]
+    leaves = [t.clone().requires_grad_(True) for t in data[0][:5]]
+    dH = data[0][5].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):       # warm-up outside the capture (library load, LDS attributes, allocator)
+        for _ in range(2):
+            for t in leaves:
+                t.grad = None
+            exp_op(*leaves, chunk_size=128).backward(dH)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    for t in leaves:
+        t.grad = None
+    with torch.cuda.graph(graph):
+        H_static = exp_op(*leaves, chunk_size=128)
+        H_static.backward(dH)
+    for rep in (1, 2, 0, 1):
+        with torch.no_grad():
+            for t, new in zip(leaves, data[rep][:5]):
+                t.copy_(new)
+            dH.copy_(data[rep][5])
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(["H", "dQ", "dK", "dV", "dI", "dF"], [H_static] + [t.grad for t in leaves], refs[rep]):
+            assert torch.equal(got, ref), f"{name}, replay with data set {rep}"
+        eager(data[(rep + 1) % 3])      # the program's own eager work between replays
+
+
 # ------------------------------------------------------------------------------------------ size-independent properties
 def test_state_passing_and_exact_value_scaling_at_full_size():
     exp_op, *_ = _ops()
