@@ -140,9 +140,10 @@ size_t mlstm_hip_chunkwise_fw_workspace_bytes(int B, int NH, int S, int DHQK, in
  *   c0,n0,m0: initial states or NULL (all three NULL together; m0 ignored for the sig gate).
  *   H (B,NH,S,DHHV) in dtype_qkv.  n_out, m_out: optional fp32 (B,NH,S) per-row normaliser max(|den|,floor)
  *   and stabiliser (NULL to skip).  c_last,n_last,m_last: optional fp32 last states (NULL to skip).
- *   With c_last given, the state scan carries the gated values as a 16-bit head plus a 16-bit remainder, so c_last
- *   is accurate to ~1e-5 relative; with c_last NULL it rounds them once (as the replaced kernels do), which is a
- *   fifth faster and changes H only within the tolerance of its 16-bit operands.
+ *   With c_last given, the state scan carries the gated values as a 16-bit head plus a 16-bit remainder in every
+ *   chunk that still weighs at least 2^-8 in the last state, so c_last is accurate to ~1e-5 relative; with c_last
+ *   NULL it rounds them once (as the replaced kernels do), which is up to a fifth faster and changes H only within
+ *   the tolerance of its 16-bit operands.
  *   MLSTM_PATH_FUSED takes bf16 only.
  *   normalize applies to the sig gate only (0: H is the bare numerator).
  */

@@ -278,8 +278,8 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   sa.f16 = f16;
   {
     ProfileScope ps("scan_fw", st);
-    // The bf16 head + remainder split of the value operand only serves the fp32 last state (1e-5 instead of 1.5e-3
-    // relative); the chunk states are rounded to bf16 anyway, so a call that returns no last state skips it.
+    // The head + remainder split of the value operand only serves the fp32 last state (1e-5 instead of 1.5e-3
+    // relative); the chunk states are rounded to 16 bits anyway, so a call that returns no last state skips it.
     if (const char* e = mlstm::launch_scan(sa, BH, /*hilo=*/c_last != nullptr, st)) return fail(e);
   }
   if (check_launch("scan_fw")) return 1;

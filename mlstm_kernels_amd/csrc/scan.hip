@@ -41,6 +41,11 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 #define SCAN_WPE(HILO_, WCOLS_) ((WCOLS_) == 64 && (HILO_) ? 1 : 2)
 // WCOLS = value columns per wave (64 or 32): with 32 a 128 x 128 tile takes eight waves, two per SIMD, each with
 // half the staging work and half the accumulators.
+template <bool V>
+struct BoolTag {
+  static constexpr bool value = V;
+};
+
 template <int RT, int WT, bool HILO, int PS, int WCOLS, bool F16>
 __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     __attribute__((amdgpu_waves_per_eu(SCAN_WPE(HILO, WCOLS), SCAN_WPE(HILO, WCOLS)))) void scan_kernel(ScanArgs a) {
@@ -142,6 +147,35 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   };
 
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
+  // The remainder of the value operand serves the last state only, and chunk c enters the last state with the weight
+  // W_c = product of the decay factors of the chunks after it (<= 1, non-increasing towards the start).  Chunks whose
+  // weight is below 2^-8 are accumulated without the remainder: their rounding (2^-9 relative) then reaches the last
+  // state at 2^-17 of its scale.  c_lo = first chunk that carries the remainder; every wave computes it for itself.
+  int c_lo = 0;
+  if constexpr (HILO) {
+    if (!a.backward) {
+      float carry = 1.f;
+      int cnt = 0;
+      for (int base = 0; base < NC; base += kWave) {
+        const int cc = NC - 1 - (base + lane);                       // walking from the last chunk towards the first
+        const float gv = cc >= 0 ? a.gbar[(size_t)bh * NC + cc] : 0.f;
+        float incl = gv;                                            // inclusive prefix product over the lanes
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+          const float up = __shfl_up(incl, o);
+          if (lane >= o) incl *= up;
+        }
+        float excl = __shfl_up(incl, 1);
+        if (lane == 0) excl = 1.f;
+        const bool need = cc >= 0 && carry * excl >= 0.00390625f;    // W_cc >= 2^-8
+        const int n_need = __popcll(__ballot(need));
+        cnt += n_need;
+        if (n_need < kWave) break;                                   // weights only fall from here on
+        carry *= __shfl(incl, kWave - 1);
+      }
+      c_lo = __builtin_amdgcn_readfirstlane(NC - cnt);
+    }
+  }
   // row scales of the first chunk straight into the table, those of the second chunk into the prefetch register
   {
     const int t = c_first * kChunk + srow;
@@ -167,6 +201,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     }
     // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split); partial sums of sum_j abar_j k_j
     const float* scur = scl + (it & 1) * kChunk + piece * PS;  // written while the previous chunk was staged
+    const bool with_lo = HILO && c >= c_lo;                    // uniform over the workgroup
     if (piece == 0 && tid < kChunk) {
       // the next chunk's row scales (fetched two chunks ahead) into the other half of the table
       const int t = (c + c_step) * kChunk + srow;
@@ -214,7 +249,9 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
         if (HILO) lo[p] = pack2<F16>(e0 - lo2<F16>(hi[p]), e1 - hi2<F16>(hi[p]));
       }
       *(uint4*)(Yh + j * YS + cv * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-      if (HILO) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      if (HILO) {
+        if (with_lo) *(uint4*)(Yl + j * YS + cv * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      }
     }
     __syncthreads();
     if (hit + 1 < NC * NP) prefetch(piece + 1 < NP ? c : c + c_step, piece + 1 < NP ? piece + 1 : 0);
@@ -258,33 +295,40 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
 
     const int q16 = (lane >> 4) & 1, i16 = lane & 15;
     const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
+    // two copies of the loop (with and without the remainder) rather than a branch inside it: the accumulators stay
+    // where they are either way
+    auto multiply = [&](auto lo_tag) {
+      constexpr bool LO = decltype(lo_tag)::value;
 #pragma unroll
-    for (int js = 0; js < PS / 16; ++js) {
-      Frag A[2], Bh[NBW], Bl[NBW];
+      for (int js = 0; js < PS / 16; ++js) {
+        Frag A[2], Bh[NBW], Bl[NBW];
 #pragma unroll
-      for (int db = 0; db < 2; ++db) {
-        const uint16_t* p = Xs + (16 * js + krow) * XS + (wr * 64 + 32 * db + ncol);
-        A[db].d[0] = lds_read_tr16(p);
-        A[db].d[1] = lds_read_tr16(p + 4 * XS);
-      }
-#pragma unroll
-      for (int wb = 0; wb < NBW; ++wb) {
-        const int o = (16 * js + krow) * YS + (wc * WCOLS + 32 * wb + ncol);
-        Bh[wb].d[0] = lds_read_tr16(Yh + o);
-        Bh[wb].d[1] = lds_read_tr16(Yh + o + 4 * YS);
-        if (HILO) {
-          Bl[wb].d[0] = lds_read_tr16(Yl + o);
-          Bl[wb].d[1] = lds_read_tr16(Yl + o + 4 * YS);
+        for (int db = 0; db < 2; ++db) {
+          const uint16_t* p = Xs + (16 * js + krow) * XS + (wr * 64 + 32 * db + ncol);
+          A[db].d[0] = lds_read_tr16(p);
+          A[db].d[1] = lds_read_tr16(p + 4 * XS);
         }
-      }
-#pragma unroll
-      for (int db = 0; db < 2; ++db)
 #pragma unroll
         for (int wb = 0; wb < NBW; ++wb) {
-          mfma32<F16>(acc[db][wb], A[db], Bh[wb]);
-          if (HILO) mfma32<F16>(acc[db][wb], A[db], Bl[wb]);
+          const int o = (16 * js + krow) * YS + (wc * WCOLS + 32 * wb + ncol);
+          Bh[wb].d[0] = lds_read_tr16(Yh + o);
+          Bh[wb].d[1] = lds_read_tr16(Yh + o + 4 * YS);
+          if (LO) {
+            Bl[wb].d[0] = lds_read_tr16(Yl + o);
+            Bl[wb].d[1] = lds_read_tr16(Yl + o + 4 * YS);
+          }
         }
-    }
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+          for (int wb = 0; wb < NBW; ++wb) {
+            mfma32<F16>(acc[db][wb], A[db], Bh[wb]);
+            if (LO) mfma32<F16>(acc[db][wb], A[db], Bl[wb]);
+          }
+      }
+    };
+    if (with_lo) multiply(BoolTag<HILO>{});
+    else multiply(BoolTag<false>{});
     // ---- normaliser vector (forward, first column tile only): n = gbar n + sum_j abar_j k_j
     if (do_n && tid < RT) {
       if (piece == 0) a.nstates[((size_t)bh * NC + c) * DHQK + d_tile + tid] = nval;

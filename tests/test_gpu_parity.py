@@ -413,6 +413,20 @@ def test_chunkwise_forward_gate_regimes(f_offset, DQK):
     assert (d64(m) - ref["m_last"]).abs().max() <= 1e-3
 
 
+@pytest.mark.parametrize("f_offset", [-2.0, 1.0, 3.0, 6.0, 12.0])
+def test_last_state_accuracy_across_decay_regimes(f_offset):
+    """The forward carries the rounding remainder of the gated values only through the chunks that still weigh at
+    least 2^-8 in the last state.  From forget gates that wipe the state within a chunk (f = -2 + N(0,1)) to gates
+    that keep everything (f = 12: all 16 chunks weigh in), C_last must stay within 1e-4 of its scale -- a tenth of
+    the state tolerance and a tenth of what a single bf16 rounding of the gated values gives (about 1e-3)."""
+    exp_op, *_ = _ops()
+    q, k, v, i, f = make_qkvif(1, 2, 2048, 128, 128, seed=31, f_offset=f_offset)
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=128)
+    _, (C, n, m) = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
+    assert_state_close(C, ref["C_last"], 1e-4, f"C_last (f = {f_offset} + N(0,1))")
+    assert_state_close(n, ref["n_last"], 1e-4, "n_last")
+
+
 def test_unsupported_head_dim_fails_loudly():
     exp_op, *_ = _ops()
     for dqk in (960, 1024):
