@@ -35,6 +35,11 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 //   eight waves per tile (64 x 32 per wave), one workgroup per CU                0.46 / 0.41   <- used
 //   eight waves, two workgroups per CU (128 registers per lane)                  -    / 0.45
 //   n recurrence shared out among the column tiles by lane masks / run by every column tile    0.51 / -    (0.48 used)
+//   rows moved from global memory straight into LDS (global_load_lds_dwordx4 into a ring of four 64-position stages,
+//   three stages ahead, XOR-swizzled tiles, one barrier per stage, rows scaled in place)   0.44 / 0.45
+//     (bit-equal results; with parts switched off: loads alone 0.22, state stores 0.05, matrix work 0.10, in-place
+//      scaling 0.04, barriers 0.04 -- the parts add up instead of overlapping, and waiting less for the loads does
+//      not change the time)
 // What pays is a second instruction stream per SIMD inside the same workgroup: the phases of a chunk (staging,
 // state emission, matrix work) are serial per wave, and two waves per SIMD overlap one's LDS and conversion
 // latencies with the other's matrix instructions.
