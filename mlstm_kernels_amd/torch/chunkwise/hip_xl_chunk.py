@@ -86,7 +86,11 @@ def validate_xl_chunk_shapes(S: int, chunk_size: int) -> None:
     assert S % chunk_size == 0, f"Sequence length must be divisible by the target chunk size {chunk_size}."
 
 
-def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep, path, stride, norm=0, norm_eps=1e-6):
+def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, keep, path, stride, norm=0, norm_eps=1e-6,
+               n_out=None, m_out=None):
+    """One forward launch.  n_out / m_out: optional fp32 (B,NH,S) tensors that receive the row normaliser
+    max(|den|, floor) and the combined stabiliser (vecN_out / vecM_out of the reference's mlstm_chunkwise_fw,
+    mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:150-170)."""
     B, NH, S, DHQK = q.shape
     DHHV = v.shape[-1]
     dev = q.device
@@ -120,7 +124,7 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
         c_last = n_last = m_last = None
     rc = lib.mlstm_hip_chunkwise_fw(
         ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), ptr(c0), ptr(n0), ptr(m0),
-        ptr(H), None, None, ptr(c_last), ptr(n_last), ptr(m_last),
+        ptr(H), ptr(n_out), ptr(m_out), ptr(c_last), ptr(n_last), ptr(m_last),
         ptr(ws), ws_bytes, int(keep), B, NH, S, DHQK, DHHV, float(eps),
         dtype_code(q), dtype_code(i), _lib.GATE_SIG if siging else _lib.GATE_EXP, int(normalize), path, stride,
         norm, float(norm_eps), ptr(norm_mean), ptr(norm_rstd), current_stream_ptr(dev),

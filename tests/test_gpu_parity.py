@@ -10,6 +10,10 @@ Stated tolerances (bf16 inputs, fp32 states):
       - on EVERY element |x - ref| <= 2e-2 + 2e-2 |ref| + 1.25 * 2^-8 * A, where A is the sum of the magnitudes of all
         products entering that element (computed by the oracle in the same chunk decomposition): the first-order
         worst case of the operand roundings.  The count of offenders and the worst one are printed per tensor.
+      - against the fp64 emulation that applies the kernels' own four 16-bit roundings and nothing else
+        (tests/rounding_emulation.py; it is the oracle when the roundings are switched off), EVERY element of H, dQ, dK,
+        dV satisfies the plain bound |x - ref| <= 2e-2 + 2e-2 |ref| (measured worst: 0.87 x the bound), at the full
+        benchmark shapes too: the elements outside the bound against the exact oracle are the operand format's.
   * final C / n / m states: 1e-3 relative (max error over tensor scale, and norm-wise).
   * dI, dF: 5e-2 of the tensor scale (sums over the head dimension / the whole sequence of differences of
     bf16-rounded products; the reference's own tests allow atol 0.4 there).
@@ -544,6 +548,82 @@ def test_chunkwise_fwbw_xlstm7b_shape_training_call():
 def test_chunkwise_fwbw_xlstm7b_shape_sig():
     """The reference's sigmoid-gate benchmark shape: mLSTMsig, B=4, S=16384, non-zero initial C ~ N(0,0.1), n ~ N(0,0.1), m = 0."""
     _fwbw_case(4, 8, 16384, 256, 512, siging=True, init=True, seed=0, pairs=[(1, 4), (2, 3)])   # middle of the grid
+
+
+@pytest.mark.parametrize("kw", [
+    dict(B=2, NH=2, S=512, DQK=128, DHV=256, seed=40),
+    dict(B=1, NH=2, S=1024, DQK=256, DHV=512, seed=41, init=True),
+    dict(B=1, NH=2, S=512, DQK=64, DHV=128, seed=42, siging=True, init=True),
+    dict(B=1, NH=2, S=512, DQK=128, DHV=64, seed=43, siging=True, normalize=False),
+    dict(B=2, NH=2, S=512, DQK=128, DHV=256, seed=44, dtype=torch.float16),
+    dict(B=4, NH=8, S=16384, DQK=256, DHV=512, seed=0, pairs=[(0, 0), (3, 7)]),
+    dict(B=16, NH=8, S=4096, DQK=256, DHV=512, seed=0, pairs=[(0, 7), (15, 0)]),
+    dict(B=64, NH=8, S=1024, DQK=256, DHV=512, seed=0, pairs=[(0, 0), (63, 7)]),
+    dict(B=4, NH=8, S=16384, DQK=256, DHV=512, seed=0, siging=True, init=True, pairs=[(1, 4), (3, 7)]),
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items() if k not in ("pairs", "seed")))
+def test_chunkwise_every_element_within_tolerance_of_the_rounding_emulation(kw, kernel_variant):
+    FRAC_EMUL, WORST_EMUL = 0.0, 1.0
+    """H, dQ, dK, dV of the training call against the fp64 emulation that rounds the same four operands the kernels
+    round (gated score blocks, chunk states, the scans' scaled value rows, the outputs) and nothing else
+    (tests/rounding_emulation.py; without the roundings it is the oracle, checked on the CPU): EVERY element inside
+    |x - ref| <= 2e-2 + 2e-2 |ref|, no allowance.  The elements that miss this bound against the exact oracle in the
+    other tests are therefore the 16-bit operand format's, not the kernels'.  The row normalisers are held to fp32
+    summation accuracy first (a denominator whose terms nearly cancel cannot be more accurate than that in fp32, and
+    the whole row scales with it), then handed to the emulation.  Split path, every state stride."""
+    import rounding_emulation as R
+
+    if not kernel_variant.startswith("split"):
+        pytest.skip("the emulation groups the products like the split path")
+    stride = int(kernel_variant.split("-")[1])
+    kw = dict(kw)
+    B, NH, S, DQK, DHV = (kw.pop(n) for n in ("B", "NH", "S", "DQK", "DHV"))
+    siging, normalize, init = kw.pop("siging", False), kw.pop("normalize", True), kw.pop("init", False)
+    dtype, seed = kw.pop("dtype", torch.bfloat16), kw.pop("seed")
+    pairs = kw.pop("pairs", None) or [(b, h) for b in range(B) for h in range(NH)]
+    exp_op, sig_op, *_ = _ops()
+    gpu_gen = torch.Generator(device=DEV).manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gpu_gen)
+    q, k, v, dH = rn(B, NH, S, DQK).to(dtype), rn(B, NH, S, DQK).to(dtype), rn(B, NH, S, DHV).to(dtype), rn(B, NH, S, DHV).to(dtype)
+    i, f = rn(B, NH, S), 3 + rn(B, NH, S)
+    c0 = n0 = m0 = None
+    if init:
+        c0, n0, m0 = 0.1 * rn(B, NH, DQK, DHV), 0.1 * rn(B, NH, DQK), torch.zeros(B, NH, 1, device=DEV)
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, i, f)]
+    okw = dict(c_initial=c0, n_initial=n0, m_initial=m0, return_last_states=False, chunk_size=128)
+    H = sig_op(*leaves, normalize=normalize, **okw) if siging else exp_op(*leaves, **okw)
+    H.backward(dH)
+    # the kernels' own row normalisers (vecN_out of the reference's forward), from one more forward launch
+    from mlstm_kernels_amd import _lib
+    from mlstm_kernels_amd.torch.chunkwise import hip_xl_chunk as X
+
+    track_n = not (siging and not normalize)
+    _, qb, kb, vb, ib, fb, c0f, n0f, m0f = X._prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
+    n_kernel = torch.empty(B, NH, S, dtype=torch.float32, device=DEV)
+    X._fw_launch(qb, kb, vb, ib, fb, c0f, n0f, m0f, 1e-6, siging, normalize, False, False, _lib.PATH_SPLIT, stride,
+                 n_out=n_kernel)
+    rnd = R.rounder(dtype)
+    results = []
+    for (b, h) in pairs:
+        sl = lambda t: None if t is None else d64(t[b:b + 1, h:h + 1])
+        args = (sl(q), sl(k), sl(v), sl(i), sl(f))
+        ekw = dict(stride=stride, siging=siging, normalize=normalize, rnd=rnd)
+        nk = None
+        if track_n:
+            # a denominator is a sum of up to 128 * stride + DHQK fp32 terms: the kernel's and the emulation's agree to
+            # a few units of fp32 roundoff of the magnitude sum of those terms
+            own = R.chunkwise_fw_rounded(*args, sl(c0), sl(n0), sl(m0), **ekw)
+            nk = sl(n_kernel)
+            excess = (nk - own["nmax_own"]).abs() - (2e-6 * own["den_abs"] + 1e-6 * own["nmax_own"])
+            assert float(excess.max()) <= 0, f"row normaliser (b={b},h={h}): off by {float(excess.max()):.3e} more than fp32 summation allows"
+        eH = R.chunkwise_fw_rounded(*args, sl(c0), sl(n0), sl(m0), nmax_given=nk, **ekw)["H"]
+        eQ, eK, eV = R.chunkwise_bw_rounded(*args, sl(dH), sl(c0), sl(n0), sl(m0), nmax_given=nk, **ekw)
+        got = [H, leaves[0].grad, leaves[1].grad, leaves[2].grad]
+        for name, x, r in zip(["H", "dQ", "dK", "dV"], got, [eH, eQ, eK, eV]):
+            bad, worst = report_offenders(x[b:b + 1, h:h + 1], r, f"{name}(b={b},h={h}) vs emulation")
+            results.append((f"{name}(b={b},h={h})", bad, worst))
+    fails = [f"{n}: {bad:.2e} of the elements outside 2e-2/2e-2 of the emulation, worst {worst:.2f} x the bound"
+             for n, bad, worst in results if bad > FRAC_EMUL or worst > WORST_EMUL]
+    assert not fails, "; ".join(fails)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

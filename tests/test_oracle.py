@@ -274,3 +274,41 @@ def test_head_normalize_matches_library_routine_and_autograd(spec):
     assert O.head_normalize(x, "none") is x
     with pytest.raises(ValueError):
         O.head_normalize(x, "batch")
+
+
+# ---------------------------------------------------------------- the rounding emulation used by the GPU tests
+@pytest.mark.parametrize("stride", [1, 2, 4])
+@pytest.mark.parametrize("siging,normalize,init", [(False, True, False), (False, True, True), (True, True, True),
+                                                   (True, False, False)])
+def test_rounding_emulation_without_rounding_is_the_oracle(stride, siging, normalize, init):
+    """tests/rounding_emulation.py restates the chunkwise forward and backward with explicit rounding points and its
+    own grouping (scans in chunks of 128, outputs per window of `stride` chunks).  With the identity as rounding
+    function it must reproduce the oracle's H, row normaliser, dQ, dK and dV to fp64 accuracy."""
+    sys_path_has_tests()
+    import rounding_emulation as R
+
+    q, k, v, i, f = make_inputs(B=1, NH=2, S=512, DQK=16, DHV=24, seed=31)
+    g = torch.Generator().manual_seed(32)
+    dH = torch.randn(1, 2, 512, 24, generator=g, dtype=torch.float64)
+    c0 = n0 = m0 = None
+    if init:
+        c0 = 0.1 * torch.randn(1, 2, 16, 24, generator=g, dtype=torch.float64)
+        n0 = 0.1 * torch.randn(1, 2, 16, generator=g, dtype=torch.float64)
+        m0 = torch.zeros(1, 2, 1, dtype=torch.float64)
+    fw = O.chunkwise_fw(q, k, v, i, f, c0, n0, m0, chunk_size=64, siging=siging, normalize=normalize)
+    bw = O.chunkwise_bw(q, k, v, i, f, dH, c0, n0, m0, chunk_size=64, siging=siging, normalize=normalize)
+    em = R.chunkwise_fw_rounded(q, k, v, i, f, c0, n0, m0, stride=stride, siging=siging, normalize=normalize)
+    dQ, dK, dV = R.chunkwise_bw_rounded(q, k, v, i, f, dH, c0, n0, m0, stride=stride, siging=siging, normalize=normalize)
+    assert torch.allclose(em["H"], fw["H"], rtol=1e-9, atol=1e-10)
+    assert torch.allclose(em["nmax"], fw["n_out"], rtol=1e-9, atol=1e-12)
+    for name, x, r in zip(["dQ", "dK", "dV"], [dQ, dK, dV], bw[:3]):
+        assert torch.allclose(x, r, rtol=1e-8, atol=1e-9), name
+
+
+def sys_path_has_tests():
+    import os
+    import sys
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    if here not in sys.path:
+        sys.path.insert(0, here)
