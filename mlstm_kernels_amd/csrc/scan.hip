@@ -40,6 +40,13 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 //     (bit-equal results; with parts switched off: loads alone 0.22, state stores 0.05, matrix work 0.10, in-place
 //      scaling 0.04, barriers 0.04 -- the parts add up instead of overlapping, and waiting less for the loads does
 //      not change the time)
+//   two LDS buffers and two register sets, one barrier per chunk: the rows of chunk c+1 are scaled and written into
+//   one buffer while chunk c is multiplied out of the other, chunk c+3 is requested meanwhile (unpadded swizzled
+//   tiles, 141 KB)                                                0.37 / 0.36 without the n recurrence, 0.44 with it
+//     (bit-equal states.  Per chunk a CU spends about 1500 cycles on LDS traffic, 1000 per SIMD on matrix
+//      instructions and 1000 per SIMD on the conversion arithmetic of the staging; with two waves per SIMD these
+//      mostly add up, whatever the order they are issued in: 2.2 us per chunk even at B = 1, where nothing else
+//      uses the memory system)
 // What pays is a second instruction stream per SIMD inside the same workgroup: the phases of a chunk (staging,
 // state emission, matrix work) are serial per wave, and two waves per SIMD overlap one's LDS and conversion
 // latencies with the other's matrix instructions.
