@@ -4,7 +4,10 @@
 (``"hip"``) and token-loop kernels (``"native_sequence__hip"``).  Unknown names raise ``ValueError``.
 
 ``register_mlstm_kernel`` / ``register_mlstm_step_kernel`` / ``register_mlstm_sequence_kernel`` let a host
-application add further callables under its own names (the package itself ships HIP kernels only)."""
+application add further callables under its own names (the package itself ships HIP kernels only).
+``use_reference_kernel_names()`` additionally answers to the reference's own Triton names, so that a configuration
+written for NX-AI/mlstm_kernels (e.g. ``chunkwise_kernel="chunkwise--triton_xl_chunk"``, ``step_kernel="triton"``)
+selects the HIP kernels unchanged."""
 from __future__ import annotations
 
 from collections.abc import Callable
@@ -46,6 +49,25 @@ def register_mlstm_step_kernel(name: str, fn: Callable) -> None:
 
 def register_mlstm_sequence_kernel(name: str, fn: Callable) -> None:
     _extra_sequence[name] = fn
+
+
+# reference name -> name here (mlstm_kernels/torch/chunkwise/__init__.py:9-15, recurrent/__init__.py:13-24)
+_REFERENCE_CHUNKWISE = {"chunkwise--triton_xl_chunk": "chunkwise--hip_xl_chunk",
+                        "chunkwise--triton_xl_chunk_siging": "chunkwise--hip_xl_chunk_siging"}
+_REFERENCE_STEP = {"triton": "hip"}
+_REFERENCE_SEQUENCE = {"native_sequence__triton": "native_sequence__hip"}
+
+
+def use_reference_kernel_names() -> None:
+    """Opt-in: registers the HIP kernels under the reference's Triton kernel names as well (the TFLA chunkwise
+    kernels, the fused step and the step-fused sequence kernel -- the ones this package replaces).  The reference's
+    other names (native_*, limit_chunk, parallel--*) stay unknown and raise ``ValueError``: there is no fallback."""
+    for ref, own in _REFERENCE_CHUNKWISE.items():
+        register_mlstm_kernel(ref, get_mlstm_kernel(own))
+    for ref, own in _REFERENCE_STEP.items():
+        register_mlstm_step_kernel(ref, get_mlstm_step_kernel(own))
+    for ref, own in _REFERENCE_SEQUENCE.items():
+        register_mlstm_sequence_kernel(ref, get_mlstm_sequence_kernel(own))
 
 
 def get_available_mlstm_kernels() -> list[str]:

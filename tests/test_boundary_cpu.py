@@ -228,3 +228,36 @@ def test_pad_zeros_wrapper(S):
     torch.testing.assert_close(H, H_ref, rtol=1e-8, atol=1e-8)
     with pytest.raises(AssertionError):
         wrap_chunkwise__pad_zeros(O.mlstm_chunkwise__native_custbw, q=q, k=k, v=v, f=f, i=i, return_last_states=True)
+
+
+def test_reference_kernel_names_are_opt_in_aliases():
+    """A configuration written for the reference (its Triton kernel names) selects the HIP kernels once
+    use_reference_kernel_names() has been called; before that the names are unknown, and the reference's other
+    kernels (native, limit_chunk, parallel) stay unknown afterwards: nothing falls back to another implementation."""
+    import mlstm_kernels_amd.torch as T
+
+    saved = ({m: dict(e) for m, e in T._extra_kernels.items()}, dict(T._extra_step), dict(T._extra_sequence))
+    before = (set(get_available_mlstm_kernels()), set(get_available_mlstm_step_kernels()),
+              set(get_available_mlstm_sequence_kernels()))
+    try:
+        with pytest.raises(ValueError):
+            get_mlstm_kernel("chunkwise--triton_xl_chunk")
+        T.use_reference_kernel_names()
+        assert get_mlstm_kernel("chunkwise--triton_xl_chunk") is get_mlstm_kernel("chunkwise--hip_xl_chunk")
+        assert get_mlstm_kernel("chunkwise--triton_xl_chunk_siging") is get_mlstm_kernel("chunkwise--hip_xl_chunk_siging")
+        assert get_mlstm_step_kernel("triton") is get_mlstm_step_kernel("hip")
+        assert get_mlstm_sequence_kernel("native_sequence__triton") is get_mlstm_sequence_kernel("native_sequence__hip")
+        cfg = mLSTMBackendConfig(chunkwise_kernel="chunkwise--triton_xl_chunk", sequence_kernel="native_sequence__triton",
+                                 step_kernel="triton", chunk_size=128, mode="inference")
+        backend = mLSTMBackend(cfg)
+        assert backend.chunkwise_kernel_fn is get_mlstm_kernel("chunkwise--hip_xl_chunk")
+        # exactly these four names were added (other tests may have registered stand-ins of their own before)
+        assert set(get_available_mlstm_kernels()) - before[0] == {"chunkwise--triton_xl_chunk", "chunkwise--triton_xl_chunk_siging"}
+        assert set(get_available_mlstm_step_kernels()) - before[1] == {"triton"}
+        assert set(get_available_mlstm_sequence_kernels()) - before[2] == {"native_sequence__triton"}
+        with pytest.raises(ValueError):
+            get_mlstm_kernel("chunkwise--triton_limit_chunk")
+    finally:
+        T._extra_kernels.clear(), T._extra_kernels.update(saved[0])
+        T._extra_step.clear(), T._extra_step.update(saved[1])
+        T._extra_sequence.clear(), T._extra_sequence.update(saved[2])
