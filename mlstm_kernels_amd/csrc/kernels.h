@@ -19,7 +19,7 @@ struct ScanArgs {
   uint16_t* states;       // bf16 fragments [BH][ceil(NC/stride)][DHHV/32][DHQK/16][64][8]
   float* final_out;       // (B,NH,DHQK,DHHV) fp32 or nullptr
   const float* n_init;    // forward: (B,NH,DHQK) or nullptr
-  float* nstates;         // forward: [BH][NC][DHQK] or nullptr (skip the n recurrence)
+  float* nstates;         // forward: [BH][NC][3][DHQK] (three partial vectors per chunk) or nullptr (skip the n recurrence)
   float* n_final;         // forward: (B,NH,DHQK) or nullptr
   int S, NC, DHQK, DHHV;
   float qk_scale, eps;
@@ -31,7 +31,7 @@ struct ScanArgs {
 struct ParHvArgs {
   const uint16_t *Q, *K, *V, *dH;  // forward uses Q,K,V; dV uses Q,K,dH
   GateBufs g;
-  const float* nstates;     // forward: n before each chunk
+  const float* nstates;     // forward: n before each chunk, [BH][NC][3][DHQK]: three partial vectors to add up
   const uint16_t* states;   // forward: C states; dV: dC states
   const float* nrow;        // dV: row normaliser (input)
   float* nrow_out;          // forward: row normaliser (output, workspace [BH][Sp])

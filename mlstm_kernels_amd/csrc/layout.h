@@ -4,7 +4,8 @@
 //   gate vectors   u, w, abar, bbar, mcomb     5 x fp32 [B*NH][NC*128]
 //   per chunk      gbar, amax, graw            3 x fp32 [B*NH][NC]
 //   stabiliser     mstates                     fp32 [B*NH][NC+1]   (index c = value before chunk c)
-//   normaliser     nstates                     fp32 [B*NH][NC][DHQK] (n before chunk c)
+//   normaliser     nstates                     fp32 [B*NH][NC][3][DHQK] (n before chunk c, as three partial vectors
+//                                              to be added up: the scan accumulates them on the matrix cores)
 //   row normaliser nrow                        fp32 [B*NH][NC*128]  max(|den|, floor), without eps
 //   chunk states   cstates                     bf16 [B*NH][ceil(NC/stride)][DHHV/32][DHQK/16][64 lanes][8]
 //                  (the state before every stride-th chunk; stride 1 keeps all of them)
@@ -67,7 +68,7 @@ inline FwWorkspace carve_fw_workspace(void* base, int B, int NH, int S, int DHQK
   w.g.amax = (float*)take(BH * NC * 4);
   w.g.mstates = (float*)take(BH * (NC + 1) * 4);
   w.g.graw = (float*)take(BH * NC * 4);
-  w.nstates = (float*)take(BH * NC * DHQK * 4);
+  w.nstates = (float*)take(BH * NC * 3 * DHQK * 4);
   w.nrow = (float*)take(BH * Sp * 4);
   w.cstates = with_states ? (uint16_t*)take(BH * NCS * (size_t)DHQK * DHHV * 2) : nullptr;
   w.bytes = off;

@@ -256,7 +256,11 @@ __device__ __forceinline__ void par_hv_body(const ParHvArgs& a, const BlockId bl
       }
     }
     if (!IS_DV) {
-      for (int d = tid; d < DHQK; d += NTH) nperm[perm16(d)] = a.nstates[((size_t)bh * NC + c) * DHQK + d];
+      // the scan hands n over as three partial vectors per chunk (their sum carries the full fp32 precision)
+      for (int d = tid; d < DHQK; d += NTH) {
+        const float* np3 = a.nstates + ((size_t)bh * NC + c) * 3 * DHQK + d;
+        nperm[perm16(d)] = (np3[0] + np3[DHQK]) + np3[2 * DHQK];
+      }
     }
   }
 
