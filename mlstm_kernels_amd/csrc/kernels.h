@@ -26,6 +26,8 @@ struct ScanArgs {
   int backward;
   int stride;             // a chunk state is kept every `stride` chunks
   int f16;                // X, Y and the state fragments are float16 instead of bfloat16
+  int part;               // set by the launcher: 0 whole sequence; 1 / 2 the two launches of a forward scan that
+                          // returns the last state (before / from the first chunk that carries the remainder)
 };
 
 struct ParHvArgs {

@@ -16,8 +16,10 @@
 // state keeps ~16 mantissa bits: a single bf16 rounding of abar*V leaves a relative error of about 1.5e-3
 // in C, above the 1e-3 the state is specified to.
 //
-// Two kernels: scan_roles_kernel (below, second) for calls that return no fp32 last state -- the training forward and
-// every backward scan -- and scan_kernel for the head + remainder split.  Same tiling, same arithmetic, same results.
+// Two kernels: scan_roles_kernel (below, second) without the remainder -- the training forward, every backward scan,
+// and of a forward that returns the fp32 last state the chunks whose rounding no longer shows in it -- and scan_kernel
+// with the head + remainder split for the rest of such a forward (two launches; the state passes from one to the
+// other in the caller's last-state buffers).  Same tiling, same arithmetic, same results.
 //
 // Workgroups are renumbered so that all tiles of one (batch, head) run on the same XCD (the hardware deals
 // consecutive workgroup ids round-robin to the 8 XCDs): the K/V rows every tile of a head re-reads then hit
@@ -57,6 +59,34 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 // emission, matrix work) are serial per wave; two waves per SIMD overlap one's LDS and conversion latencies with the
 // other's matrix instructions, and four waves in two roles keep the conversion arithmetic and the matrix
 // instructions in different waves altogether.
+// The remainder of the value operand serves the last state only, and chunk c enters the last state with the weight
+// W_c = product of the decay factors of the chunks after it (<= 1, non-increasing towards the start).  Chunks whose
+// weight is below 2^-8 are accumulated without the remainder: their rounding (2^-9 relative) then reaches the last
+// state at 2^-17 of its scale.  Returns the first chunk that carries the remainder (at most NC - 1); every wave
+// computes it for itself, and every kernel that needs it gets the same value.
+__device__ __forceinline__ int first_remainder_chunk(const float* gbar_bh, int NC, int lane) {
+  float carry = 1.f;
+  int cnt = 0;
+  for (int base = 0; base < NC; base += kWave) {
+    const int cc = NC - 1 - (base + lane);                       // walking from the last chunk towards the first
+    const float gv = cc >= 0 ? gbar_bh[cc] : 0.f;
+    float incl = gv;                                            // inclusive prefix product over the lanes
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const float up = __shfl_up(incl, o);
+      if (lane >= o) incl *= up;
+    }
+    float excl = __shfl_up(incl, 1);
+    if (lane == 0) excl = 1.f;
+    const bool need = cc >= 0 && carry * excl >= 0.00390625f;    // W_cc >= 2^-8
+    const int n_need = __popcll(__ballot(need));
+    cnt += n_need;
+    if (n_need < kWave) break;                                   // weights only fall from here on
+    carry *= __shfl(incl, kWave - 1);
+  }
+  return __builtin_amdgcn_readfirstlane(NC - cnt);
+}
+
 #define SCAN_WPE(HILO_, WCOLS_) ((WCOLS_) == 64 && (HILO_) ? 1 : 2)
 // WCOLS = value columns per wave (64 or 32): with 32 a 128 x 128 tile takes eight waves, two per SIMD, each with
 // half the staging work and half the accumulators.
@@ -116,17 +146,21 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         float v0 = 0.f;
-        if (a.init != nullptr) {
+        const float* init = a.part == 2 ? a.final_out : a.init;  // part 2 continues from the first launch's state
+        if (init != nullptr) {
           const int d = d_wave + 32 * db + 8 * (i / 4) + 4 * h + (i % 4);
           const int w = w_wave + 32 * wb + r;
-          v0 = a.init[((size_t)bh * DHQK + d) * DHHV + w];
+          v0 = init[((size_t)bh * DHQK + d) * DHHV + w];
         }
         acc[db][wb][i] = v0;
       }
     }
   const bool do_n = (a.nstates != nullptr) && by == 0;
   float nval = 0.f;
-  if (do_n && tid < RT && a.n_init != nullptr) nval = a.n_init[(size_t)bh * DHQK + d_tile + tid];
+  {
+    const float* n_init = a.part == 2 ? a.n_final : a.n_init;
+    if (do_n && tid < RT && n_init != nullptr) nval = n_init[(size_t)bh * DHQK + d_tile + tid];
+  }
 
   const uint16_t* Xg = a.X + (size_t)bh * S * DHQK + d_tile;
   const uint16_t* Yg = a.Y + (size_t)bh * S * DHHV + w_tile;
@@ -165,36 +199,16 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     }
   };
 
-  const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
-  // The remainder of the value operand serves the last state only, and chunk c enters the last state with the weight
-  // W_c = product of the decay factors of the chunks after it (<= 1, non-increasing towards the start).  Chunks whose
-  // weight is below 2^-8 are accumulated without the remainder: their rounding (2^-9 relative) then reaches the last
-  // state at 2^-17 of its scale.  c_lo = first chunk that carries the remainder; every wave computes it for itself.
+  const int c_first_all = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
+  // c_lo = first chunk that carries the remainder of the value operand
   int c_lo = 0;
   if constexpr (HILO) {
-    if (!a.backward) {
-      float carry = 1.f;
-      int cnt = 0;
-      for (int base = 0; base < NC; base += kWave) {
-        const int cc = NC - 1 - (base + lane);                       // walking from the last chunk towards the first
-        const float gv = cc >= 0 ? a.gbar[(size_t)bh * NC + cc] : 0.f;
-        float incl = gv;                                            // inclusive prefix product over the lanes
-#pragma unroll
-        for (int o = 1; o < kWave; o <<= 1) {
-          const float up = __shfl_up(incl, o);
-          if (lane >= o) incl *= up;
-        }
-        float excl = __shfl_up(incl, 1);
-        if (lane == 0) excl = 1.f;
-        const bool need = cc >= 0 && carry * excl >= 0.00390625f;    // W_cc >= 2^-8
-        const int n_need = __popcll(__ballot(need));
-        cnt += n_need;
-        if (n_need < kWave) break;                                   // weights only fall from here on
-        carry *= __shfl(incl, kWave - 1);
-      }
-      c_lo = __builtin_amdgcn_readfirstlane(NC - cnt);
-    }
+    if (!a.backward) c_lo = first_remainder_chunk(a.gbar + (size_t)bh * NC, NC, lane);
   }
+  // part 2 of a forward scan in two launches: the chunks from c_lo on, continuing from the state the first launch left
+  // in final_out / n_final (loaded above)
+  const int c_first = a.part == 2 ? c_lo : c_first_all;
+  const int NCR = a.part == 2 ? NC - c_lo : NC;  // chunks this launch runs
   // row scales of the first chunk straight into the table, those of the second chunk into the prefetch register
   {
     const int t = c_first * kChunk + srow;
@@ -205,9 +219,9 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     }
     if (tid < kChunk) scl[srow] = sc0;
   }
-  load_scales(NC > 1 ? c_first + c_step : c_first);
+  load_scales(NCR > 1 ? c_first + c_step : c_first);
   prefetch(c_first, 0);
-  for (int hit = 0; hit < NC * NP; ++hit) {
+  for (int hit = 0; hit < NCR * NP; ++hit) {
     const int it = hit / NP, piece = hit % NP;
     const int c = c_first + it * c_step;
     // The decay factors come from LDS, a block of chunks at a time: read straight from global memory inside the
@@ -215,7 +229,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     // work would wait for the whole prefetch in every iteration.
     if (piece == 0 && (it & (kGBlock - 1)) == 0) {
       __syncthreads();
-      for (int k = tid; k < kGBlock && it + k < NC; k += NT) gl[k] = a.gbar[(size_t)bh * NC + c + k * c_step];
+      for (int k = tid; k < kGBlock && it + k < NCR; k += NT) gl[k] = a.gbar[(size_t)bh * NC + c + k * c_step];
       // visible after the barrier that follows the staging below
     }
     // ---- registers -> LDS (Y rows scaled in fp32, then rounded / split); partial sums of sum_j abar_j k_j
@@ -224,7 +238,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
     if (piece == 0 && tid < kChunk) {
       // the next chunk's row scales (fetched two chunks ahead) into the other half of the table
       const int t = (c + c_step) * kChunk + srow;
-      float sn = (it + 1 < NC && t < S) ? s_raw : 0.f;
+      float sn = (it + 1 < NCR && t < S) ? s_raw : 0.f;
       if (a.backward) {
         sn *= a.qk_scale;
         if (a.nrow != nullptr) sn /= (s_nrm + a.eps);
@@ -273,7 +287,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
       }
     }
     __syncthreads();
-    if (hit + 1 < NC * NP) prefetch(piece + 1 < NP ? c : c + c_step, piece + 1 < NP ? piece + 1 : 0);
+    if (hit + 1 < NCR * NP) prefetch(piece + 1 < NP ? c : c + c_step, piece + 1 < NP ? piece + 1 : 0);
     if (piece == 0) load_scales(c + 2 * c_step);
 
     // ---- emit the state before this chunk's update as bf16 operand fragments, at the kept boundaries only: forward
@@ -443,7 +457,8 @@ __device__ __forceinline__ Frag scan_tr_frag(const uint16_t* tile, int k0, const
 // instructions, which would make the compiler keep those accumulators in scratch memory).
 template <int RT, int WT, bool F16, int NDB>
 __device__ __forceinline__ void scan_consumer(const ScanArgs& a, const uint16_t* bufs, const float* gl, const uint16_t* nB,
-                                              int wave, int lane, int bh, int d_tile, int w_tile, int c_lo) {
+                                              int wave, int lane, int bh, int d_tile, int w_tile, int n_run) {
+  constexpr int c_lo = 0;  // (no remainder operand in this kernel)
   constexpr bool HILO = false;
   constexpr int WC = WT / 32;
   constexpr int PS = HILO ? 64 : 128;
@@ -451,7 +466,7 @@ __device__ __forceinline__ void scan_consumer(const ScanArgs& a, const uint16_t*
   constexpr int XELEMS = PS * RT, YELEMS = PS * WT;
   constexpr int BUF = XELEMS + YELEMS * (HILO ? 2 : 1);
   const int DHQK = a.DHQK, DHHV = a.DHHV, NC = a.NC;
-  const int total = NC * NP;
+  const int total = n_run * NP;  // n_run: chunks this launch runs
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
   constexpr bool WITH_N = NDB >= 0;
   constexpr int DB = WITH_N ? NDB : 0;
@@ -624,7 +639,10 @@ __global__ __launch_bounds__(128 * (RT / 64) * (WT / 32)) void scan_roles_kernel
   const int d_tile = blk.x * RT, w_tile = blk.y * WT;
   const int DHQK = a.DHQK, DHHV = a.DHHV, S = a.S, NC = a.NC;
   const size_t Sp = (size_t)NC * kChunk;
-  const int total = NC * NP;
+  // part 1 of a forward scan in two launches: only the chunks before the first one that carries the remainder of the
+  // value operand; the state reached there is handed over in final_out / n_final
+  const int n_run = a.part == 1 ? first_remainder_chunk(a.gbar + (size_t)bh * NC, NC, lane) : NC;
+  const int total = n_run * NP;
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
 
   constexpr int c_lo = 0;  // (no remainder operand in this kernel)
@@ -743,10 +761,10 @@ __global__ __launch_bounds__(128 * (RT / 64) * (WT / 32)) void scan_roles_kernel
     // (the prefetches are unconditional, past the end the last piece is fetched again: a conditional prefetch makes
     // the compiler keep the register sets in scratch memory across the loop back-edge)
     MLSTM_SCAN_PREFETCH(0, 0)
-    MLSTM_SCAN_PREFETCH(1, min(1, total - 1))
+    MLSTM_SCAN_PREFETCH(1, max(min(1, total - 1), 0))
     __syncthreads();  // scale table visible
     MLSTM_SCAN_STAGE(0, 0, 0)
-    MLSTM_SCAN_PREFETCH(0, min(2, total - 1))
+    MLSTM_SCAN_PREFETCH(0, max(min(2, total - 1), 0))
 
     // one piece p of parity PAR (its LDS buffer); the pieces p+1 and p+3 use the other buffer and register set
 #define MLSTM_SCAN_BODY(PAR, OTHER, p_)                                                                          \
@@ -787,11 +805,11 @@ __global__ __launch_bounds__(128 * (RT / 64) * (WT / 32)) void scan_roles_kernel
     // 0 and 1 carry it for the first and the second 32 rows
     const bool with_n = (a.nstates != nullptr) && blk.y == 0;
     if (with_n && wave % WC == 0)
-      scan_consumer<RT, WT, F16, 0>(a, bufs, gl, nB, wave, lane, bh, d_tile, w_tile, c_lo);
+      scan_consumer<RT, WT, F16, 0>(a, bufs, gl, nB, wave, lane, bh, d_tile, w_tile, n_run);
     else if (with_n && wave % WC == 1)
-      scan_consumer<RT, WT, F16, 1>(a, bufs, gl, nB, wave, lane, bh, d_tile, w_tile, c_lo);
+      scan_consumer<RT, WT, F16, 1>(a, bufs, gl, nB, wave, lane, bh, d_tile, w_tile, n_run);
     else
-      scan_consumer<RT, WT, F16, -1>(a, bufs, gl, nB, wave, lane, bh, d_tile, w_tile, c_lo);
+      scan_consumer<RT, WT, F16, -1>(a, bufs, gl, nB, wave, lane, bh, d_tile, w_tile, n_run);
   }
 }
 
@@ -811,20 +829,35 @@ static const char* launch_scan_roles_t(const ScanArgs& a, int BH, hipStream_t st
   return a.f16 ? launch_scan_roles_f<RT, WT, true>(a, BH, stream) : launch_scan_roles_f<RT, WT, false>(a, BH, stream);
 }
 
-const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream) {
+const char* launch_scan(const ScanArgs& a_in, int BH, bool hilo, hipStream_t stream) {
+  ScanArgs a = a_in;
+  a.part = 0;
   if (a.DHQK % 64 != 0 || a.DHHV % 64 != 0) return "scan: DHQK and DHHV must be multiples of 64";
   if (a.stride < 1 || a.stride > kMaxStateStride) return "scan: state stride out of range";
   const bool r128 = a.DHQK % 128 == 0, w128 = a.DHHV % 128 == 0;
+  auto roles = [&]() -> const char* {
+    if (r128 && w128) return launch_scan_roles_t<128, 128>(a, BH, stream);
+    if (r128) return launch_scan_roles_t<128, 64>(a, BH, stream);
+    if (w128) return launch_scan_roles_t<64, 128>(a, BH, stream);
+    return launch_scan_roles_t<64, 64>(a, BH, stream);
+  };
   if (hilo) {
+    // Two launches (forward only): the chunks whose rounding no longer shows in the last state go through the faster
+    // kernel without the remainder operand, which leaves its state in final_out / n_final; the kernel with the
+    // remainder continues from there.  Both find the chunk where they meet from the decay factors alone.
+    if (a.final_out == nullptr || a.backward) return "scan: the remainder split serves the forward last state only";
+    const bool two = a.nstates == nullptr || a.n_final != nullptr;  // n needs its hand-over buffer too
+    if (two) {
+      a.part = 1;
+      if (const char* e = roles()) return e;
+      a.part = 2;
+    }
     if (r128 && w128) return launch_scan_t<128, 128, true>(a, BH, stream);
     if (r128) return launch_scan_t<128, 64, true>(a, BH, stream);
     if (w128) return launch_scan_t<64, 128, true>(a, BH, stream);
     return launch_scan_t<64, 64, true>(a, BH, stream);
   }
-  if (r128 && w128) return launch_scan_roles_t<128, 128>(a, BH, stream);
-  if (r128) return launch_scan_roles_t<128, 64>(a, BH, stream);
-  if (w128) return launch_scan_roles_t<64, 128>(a, BH, stream);
-  return launch_scan_roles_t<64, 64>(a, BH, stream);
+  return roles();
 }
 
 }  // namespace mlstm
