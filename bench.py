@@ -61,6 +61,7 @@ FLOPS_PER_TOKEN_HEAD = {
 # the fused sequential kernels do the work of a scan plus the chunk-parallel kernel that follows it
 FLOPS_PER_TOKEN_HEAD["fused_fw"] = FLOPS_PER_TOKEN_HEAD["scan_fw"] + FLOPS_PER_TOKEN_HEAD["par_h"]
 FLOPS_PER_TOKEN_HEAD["fused_dv"] = FLOPS_PER_TOKEN_HEAD["scan_bw"] + FLOPS_PER_TOKEN_HEAD["par_dv"]
+FLOPS_PER_TOKEN_HEAD["scan_fw_recompute"] = FLOPS_PER_TOKEN_HEAD["scan_fw"]   # the state scan run again in the backward
 FLOPS_FW = 4 * DHQK * DHHV + CHUNK * (DHQK + DHHV)
 FLOPS_BW = 8 * DHQK * DHHV + CHUNK * (3 * DHQK + 2 * DHHV)
 assert sum(FLOPS_PER_TOKEN_HEAD[n] for n in ("fused_fw", "fused_dv", "par_dqdk")) == FLOPS_FW + FLOPS_BW
@@ -188,7 +189,7 @@ def main():
     stride = args.state_stride or _lib.default_state_stride(B, NH, S, DHQK, DHHV)
 
     def run_config(Bc, Sc, steps, warmup, sig=False, init=False, backward=True, profile_steps=3, head_norm="none",
-                   dtype=torch.bfloat16, last_states=False):
+                   dtype=torch.bfloat16, last_states=False, recompute=False):
         """Times `steps` passes of one configuration (median of per-step HIP-event times, caches flushed before every
         step), then profiles `profile_steps` further passes kernel by kernel."""
         q = rn(Bc, NH, Sc, DHQK).to(dtype).requires_grad_(backward)
@@ -198,6 +199,8 @@ def main():
         f = (3 + rn(Bc, NH, Sc)).requires_grad_(backward)
         dH = rn(Bc, NH, Sc, DHHV).to(dtype)
         kw = dict(chunk_size=CHUNK, autocast_kernel_dtype=dtype, head_norm=head_norm, return_last_states=last_states, **intra)
+        if recompute:
+            kw["recompute_states_in_bw"] = True   # the reference's default saved-state policy
         if init:
             kw.update(c_initial=0.1 * rn(Bc, NH, DHQK, DHHV), n_initial=0.1 * rn(Bc, NH, DHQK),
                       m_initial=torch.zeros(Bc, NH, 1, device=dev))
@@ -294,6 +297,7 @@ def main():
         for tag, cfg in (("exp_fwbw_B16_S4096", dict(Bc=16, Sc=4096)), ("exp_fwbw_B64_S1024", dict(Bc=64, Sc=1024)),
                          ("sig_fwbw_B4_S16384_init", dict(Bc=4, Sc=16384, sig=True, init=True)),
                          ("exp_fwbw_B4_S16384_float16", dict(Bc=4, Sc=16384, dtype=torch.float16)),
+                         ("exp_fwbw_B4_S16384_recompute_states_in_bw", dict(Bc=4, Sc=16384, recompute=True)),
                          ("exp_fw_B4_S16384", dict(Bc=4, Sc=16384, backward=False)),
                          ("exp_fw_B4_S16384_last_states", dict(Bc=4, Sc=16384, backward=False, last_states=True)),
                          ("exp_fw_B4_S16384_head_norm_layer", dict(Bc=4, Sc=16384, backward=False, head_norm="layer")),

@@ -157,6 +157,25 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
                            int head_norm, float norm_eps, float* norm_mean, float* norm_rstd, void* stream);
 
 /*
+ * Saved-state policy of the reference (recompute_states_in_bw, mlstm_kernels/torch/chunkwise/triton_xl_chunk/fwbw.py:45-62
+ * and bw.py:75-95: the forward keeps no chunk states and the backward runs the state recurrence again).  The chunk
+ * states are the last and by far the largest part of the forward workspace; a caller that wants to hold less memory
+ * between forward and backward keeps only the first mlstm_hip_chunkwise_fw_saved_bytes() bytes of it (gate vectors,
+ * normaliser states, row normalisers: independent of state_stride), and before the backward copies them to the start
+ * of a full-size workspace and calls mlstm_hip_chunkwise_recompute_states, which runs the forward state scan again
+ * and writes the chunk states behind them (k, v, c0, dtype_qkv, state_stride as in the forward call; c0 NULL = zero
+ * initial state).  The workspace is then what mlstm_hip_chunkwise_bw expects.  The recomputed states equal the
+ * forward's bit for bit when the forward returned no last state (c_last NULL); a forward that returned it carried a
+ * remainder of the value operand in its late chunks, and the recomputed states of those chunks differ from the
+ * forward's by one 16-bit rounding of that operand.
+ */
+size_t mlstm_hip_chunkwise_fw_saved_bytes(int B, int NH, int S, int DHQK, int DHHV);
+int mlstm_hip_chunkwise_recompute_states(const void* k, const void* v, const float* c0,
+                                         void* workspace, size_t workspace_bytes,
+                                         int B, int NH, int S, int DHQK, int DHHV,
+                                         int dtype_qkv, int state_stride, void* stream);
+
+/*
  * Backward of the fused head norm: dX = rstd * (dY - mean_D(dY) - Y * mean_D(dY * Y)) for MLSTM_NORM_LAYER,
  * dX = rstd * (dY - Y * mean_D(dY * Y)) for MLSTM_NORM_RMS, per row of D = 64, 128, 256 or 512 values.
  * Replaces the autograd backward of the reference's layer_normalize / rms_normalize

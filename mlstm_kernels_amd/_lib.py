@@ -14,7 +14,7 @@ F16 = 2
 GATE_EXP, GATE_SIG = 0, 1
 PATH_AUTO, PATH_SPLIT, PATH_FUSED = 0, 1, 2
 NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 NOALLOC_SCRATCH_BYTES = 64 << 20  # MLSTM_NOALLOC_SCRATCH_BYTES of include/mlstm_hip.h
 
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
@@ -28,6 +28,8 @@ _SIGNATURES = {
     "mlstm_hip_recurrent_sequence": (_i, [_vp] * 12 + [_i, _i, _i, _i, _i, _f, _i, _i, _i, _vp]),
     "mlstm_hip_chunkwise_fw_workspace_bytes": (_sz, [_i] * 8),
     "mlstm_hip_chunkwise_fw": (_i, [_vp] * 15 + [_sz, _i] + [_i] * 5 + [_f] + [_i] * 7 + [_f, _vp, _vp] + [_vp]),
+    "mlstm_hip_chunkwise_fw_saved_bytes": (_sz, [_i] * 5),
+    "mlstm_hip_chunkwise_recompute_states": (_i, [_vp] * 4 + [_sz] + [_i] * 7 + [_vp]),
     "mlstm_hip_head_norm_bw": (_i, [_vp] * 4 + [_sz, _i, _i, _i, _vp]),
     "mlstm_hip_chunkwise_fw_noalloc": (_i, [_vp] * 14 + [_i] * 5 + [_f] + [_i] * 4 + [_vp]),
     "mlstm_hip_chunkwise_bw_workspace_bytes": (_sz, [_i] * 6),

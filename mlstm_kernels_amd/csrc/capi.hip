@@ -94,7 +94,7 @@ static bool valid_dtype(int code) { return code == MLSTM_F32 || code == MLSTM_BF
 
 extern "C" {
 
-int mlstm_hip_abi_version(void) { return 5; }
+int mlstm_hip_abi_version(void) { return 6; }
 
 int mlstm_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
@@ -324,6 +324,45 @@ int mlstm_hip_chunkwise_fw(const void* q, const void* k, const void* v, const vo
                            workspace, workspace_bytes, keep_for_backward, B, NH, S, DHQK, DHHV, eps, dtype_qkv,
                            dtype_gates, gate, normalize, path, state_stride, head_norm, norm_eps, norm_mean, norm_rstd,
                            (hipStream_t)stream);
+}
+
+size_t mlstm_hip_chunkwise_fw_saved_bytes(int B, int NH, int S, int DHQK, int DHHV) {
+  if (check_dims(B, NH, S, DHQK, DHHV)) return 0;
+  // the chunk states are carved last: without them the workspace is exactly the part in front of them
+  return mlstm::carve_fw_workspace(nullptr, B, NH, S, DHQK, DHHV, /*with_states=*/false, 1).bytes;
+}
+
+int mlstm_hip_chunkwise_recompute_states(const void* k, const void* v, const float* c0, void* workspace,
+                                         size_t workspace_bytes, int B, int NH, int S, int DHQK, int DHHV,
+                                         int dtype_qkv, int state_stride, void* stream) {
+  if (!k || !v || !workspace) return fail("mlstm_hip_chunkwise_recompute_states: null pointer argument");
+  if (const char* e = check_dims(B, NH, S, DHQK, DHHV)) return fail(e);
+  if (const char* e = check_options(MLSTM_PATH_AUTO, state_stride, DHQK, DHHV)) return fail(e);
+  if (dtype_qkv != MLSTM_BF16 && dtype_qkv != MLSTM_F16)
+    return fail("mlstm_hip_chunkwise_recompute_states: k/v must be bf16 or fp16");
+  const int stride = resolve_stride(state_stride);
+  mlstm::FwWorkspace ws = mlstm::carve_fw_workspace(workspace, B, NH, S, DHQK, DHHV, true, stride);
+  if (workspace_bytes < ws.bytes) return fail("mlstm_hip_chunkwise_recompute_states: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  mlstm::ScanArgs sa;
+  memset(&sa, 0, sizeof(sa));
+  sa.X = (const uint16_t*)k;
+  sa.Y = (const uint16_t*)v;
+  sa.scale_a = ws.g.abar;
+  sa.gbar = ws.g.gbar;
+  sa.init = c0;
+  sa.states = ws.cstates;
+  // the normaliser states in front of the chunk states are the forward's own: the recurrence of n is not run again
+  sa.S = S; sa.NC = (S + 127) / 128; sa.DHQK = DHQK; sa.DHHV = DHHV;
+  sa.qk_scale = 1.0f / sqrtf((float)DHQK);
+  sa.backward = 0;
+  sa.stride = stride;
+  sa.f16 = dtype_qkv == MLSTM_F16;
+  {
+    ProfileScope ps("scan_fw_recompute", st);
+    if (const char* e = mlstm::launch_scan(sa, B * NH, /*hilo=*/false, st)) return fail(e);
+  }
+  return check_launch("mlstm_hip_chunkwise_recompute_states");
 }
 
 int mlstm_hip_head_norm_bw(const void* dY, const void* Y, const float* rstd, void* dX, size_t rows, int D, int head_norm,

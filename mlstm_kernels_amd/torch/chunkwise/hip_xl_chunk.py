@@ -8,8 +8,10 @@ with the same argument names, defaults, return structure and shape rules
 internal chunks of 128 positions (the reference's ``chunk_size_inter``), which leaves H and the last states unchanged
 because the chunkwise formulation is exact for every chunk length.  ``chunk_size_intra`` (a multiple of 128, at most
 1024) selects how far apart the kept chunk states are, as in the reference (``save_states_every_nth_chunk`` =
-``chunk_size_intra // chunk_size_inter``); ``chunk_size_inter`` is checked and otherwise has no effect; the Triton
-tile-size and launch keywords are accepted and ignored.
+``chunk_size_intra // chunk_size_inter``); ``chunk_size_inter`` is checked and otherwise has no effect;
+``recompute_states_in_bw=True`` makes the autograd function drop the chunk states after the forward and run the state
+scan again in the backward, as the reference does (default here: ``False``, the states are kept -- the reference's
+default is ``True``); the Triton tile-size and launch keywords are accepted and ignored.
 
 Arithmetic: the matrix cores multiply bfloat16 or float16 operands -- the dtype of q after the autocast cast to
 ``autocast_kernel_dtype`` -- and accumulate in fp32; gates, stabilisers, normalisers and states are fp32.  float32
@@ -27,8 +29,9 @@ from ..utils import current_stream_ptr, dtype_code, ptr, require_gpu
 
 _IGNORED_TUNING_KWARGS = (
     "siz_b_L_parallel", "siz_b_L_loop", "siz_b_DH_parallel", "siz_b_DH_loop", "num_warps_intra", "num_warps_inter",
-    "num_stages_intra", "num_stages_inter", "recompute_states_in_bw",
+    "num_stages_intra", "num_stages_inter",
 )
+_POLICY_KWARGS = ("chunk_size_inter", "chunk_size_intra", "recompute_states_in_bw")
 _INTERNAL_CHUNK = 128
 _warned_rounding: set = set()
 
@@ -53,7 +56,7 @@ def _state_stride(tuning_kwargs: dict, who: str) -> int:
     chunk_size_intra); chunk_size_intra sets the distance between kept states, in units of 128 positions (a smaller
     value keeps a state per internal chunk)."""
     for key in tuning_kwargs:
-        if key not in _IGNORED_TUNING_KWARGS and key not in ("chunk_size_inter", "chunk_size_intra"):
+        if key not in _IGNORED_TUNING_KWARGS and key not in _POLICY_KWARGS:
             raise TypeError(f"{who}() got an unexpected keyword argument '{key}'")
     inter = tuning_kwargs.get("chunk_size_inter")
     intra = tuning_kwargs.get("chunk_size_intra")
@@ -69,6 +72,15 @@ def _state_stride(tuning_kwargs: dict, who: str) -> int:
         raise ValueError(f"chunk_size_intra must be 16, 32, 64 or a multiple of {_INTERNAL_CHUNK} up to "
                          f"{8 * _INTERNAL_CHUNK}, got {intra}")
     return intra // _INTERNAL_CHUNK
+
+
+def _recompute_states(tuning_kwargs: dict) -> bool:
+    """recompute_states_in_bw of the reference (triton_xl_chunk/fwbw.py:45,62): True = keep no chunk states between
+    forward and backward and run the state scan again in the backward.  Unlike the reference the default is False."""
+    flag = tuning_kwargs.get("recompute_states_in_bw")
+    if flag is not None and not isinstance(flag, bool):
+        raise ValueError(f"recompute_states_in_bw must be True, False or None, got {flag!r}")
+    return bool(flag)
 
 
 def _is_pow2(x: int) -> bool:
@@ -159,7 +171,8 @@ def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
     return dev, qb, kb, vb, ib, fb, c0, n0, m0
 
 
-def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, stride: int, norm: int, norm_eps: float):
+def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, stride: int, norm: int, norm_eps: float,
+               recompute: bool):
     class _HipChunkwiseFwBw(torch.autograd.Function):
         @staticmethod
         @custom_fwd(device_type="cuda", cast_inputs=autocast_kernel_dtype)
@@ -174,10 +187,19 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
                 qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw, path, stride,
                 norm, norm_eps
             )
+            c0s = None
+            if recompute and needs_bw:
+                # keep only what lies in front of the chunk states (gate vectors, normaliser states, row normalisers);
+                # the backward runs the state scan again, from the initial state when there is one
+                B_, NH_, S_, DHQK_ = qb.shape
+                saved_bytes = _lib.get_lib().mlstm_hip_chunkwise_fw_saved_bytes(B_, NH_, S_, DHQK_, vb.shape[-1])
+                if ws.numel() > saved_bytes:
+                    ws = ws[:saved_bytes].clone()
+                c0s = c0f
             if norm != _lib.NORM_NONE and needs_bw:
-                ctx.save_for_backward(qb, kb, vb, ib, fb, ws, H, norm_rstd)   # H holds the normalised rows
+                ctx.save_for_backward(qb, kb, vb, ib, fb, ws, c0s, H, norm_rstd)   # H holds the normalised rows
             else:
-                ctx.save_for_backward(qb, kb, vb, ib, fb, ws)
+                ctx.save_for_backward(qb, kb, vb, ib, fb, ws, c0s)
             ctx.cfg = (eps, q.dtype, k.dtype, v.dtype, i.dtype, f.dtype,
                        None if c0 is None else c0.dtype, n0 is not None, m0 is not None)
             H = H if out_dtype == H.dtype else H.to(out_dtype)
@@ -186,7 +208,7 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
         @staticmethod
         @custom_bwd(device_type="cuda")
         def backward(ctx, dH, dC_last, dn_last, dm_last):
-            qb, kb, vb, ib, fb, ws, *normed = ctx.saved_tensors
+            qb, kb, vb, ib, fb, ws, c0s, *normed = ctx.saved_tensors
             eps, qdt, kdt, vdt, idt, fdt, c0dt, has_n0, has_m0 = ctx.cfg
             B, NH, S, DHQK = qb.shape
             DHHV = vb.shape[-1]
@@ -194,6 +216,16 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
             lib = _lib.get_lib()
             bw_bytes = lib.mlstm_hip_chunkwise_bw_workspace_bytes(B, NH, S, DHQK, DHHV, stride)
             bws = torch.empty(bw_bytes, dtype=torch.uint8, device=dev)
+            if recompute:
+                full_bytes = lib.mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 1, path, stride)
+                full = torch.empty(full_bytes, dtype=torch.uint8, device=dev)
+                full[:ws.numel()].copy_(ws)
+                rc = lib.mlstm_hip_chunkwise_recompute_states(
+                    ptr(kb), ptr(vb), ptr(c0s), ptr(full), full_bytes, B, NH, S, DHQK, DHHV, dtype_code(qb), stride,
+                    current_stream_ptr(dev),
+                )
+                _lib.check(rc, "mlstm_hip_chunkwise_recompute_states")
+                ws = full
             if dH is None:  # only the last states are differentiated
                 dH = torch.zeros(B, NH, S, DHHV, dtype=qb.dtype, device=dev)
             dHb = dH.to(qb.dtype).contiguous()
@@ -230,16 +262,17 @@ _FWBW_CACHE: dict = {}
 
 
 def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool, kernel_path: str, stride: int,
-              head_norm: str = "none", head_norm_eps: float = 1e-6):
+              head_norm: str = "none", head_norm_eps: float = 1e-6, recompute: bool = False):
     if autocast_kernel_dtype not in (torch.float32, torch.float16, torch.bfloat16):
         raise ValueError(f"Unsupported kernel dtype {autocast_kernel_dtype}.")
     path = _lib.path_code(kernel_path)
     norm = _lib.norm_code(head_norm)
     if norm != _lib.NORM_NONE and path == _lib.PATH_FUSED:
         raise ValueError("head_norm is fused into the split kernel path only (kernel_path='auto' or 'split')")
-    key = (autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps))
+    key = (autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps), bool(recompute))
     if key not in _FWBW_CACHE:
-        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps))
+        _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps),
+                                      bool(recompute))
     return _FWBW_CACHE[key]
 
 
@@ -269,7 +302,8 @@ def mlstm_chunkwise__hip_xl_chunk(
     ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
     tail themselves, so every S >= 1 is one call.  ``kernel_path`` ("auto", "split", "fused"; not in the reference)
     selects the kernels of the value-column side.  ``chunk_size_intra`` (reference keyword) sets the distance between
-    kept chunk states.  ``head_norm`` ("none", "layer", "rms"; not in the reference's operator) fuses the multi-head
+    kept chunk states; ``recompute_states_in_bw=True`` (reference keyword) keeps none of them between forward and
+    backward.  ``head_norm`` ("none", "layer", "rms"; not in the reference's operator) fuses the multi-head
     norm that follows the cell in the xLSTM block -- the reference's ``apply_normalize(norm_specifier, x, eps)``,
     mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-64, over the DHHV columns of every row, without
     scale parameters -- into the output kernel: the returned ``H`` is then the normalised one and the un-normalised
@@ -277,7 +311,8 @@ def mlstm_chunkwise__hip_xl_chunk(
     stride = _state_stride(tuning_kwargs, "mlstm_chunkwise__hip_xl_chunk")
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
-    fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride, head_norm, head_norm_eps)
+    fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride, head_norm, head_norm_eps,
+                   _recompute_states(tuning_kwargs))
     H, c_last, n_last, m_last = fn.apply(q, k, v, i, f, c_initial, n_initial, m_initial, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last, m_last)
@@ -309,7 +344,8 @@ def mlstm_siging_chunkwise__hip_xl_chunk(
     stride = _state_stride(tuning_kwargs, "mlstm_siging_chunkwise__hip_xl_chunk")
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
-    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride, head_norm, head_norm_eps)
+    fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride, head_norm, head_norm_eps,
+                   _recompute_states(tuning_kwargs))
     H, c_last, n_last, _ = fn.apply(q, k, v, i, f, c_initial, n_initial, None, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last)

@@ -80,9 +80,15 @@ def test_shape_rules_of_the_xl_chunk_operator():
 def test_operator_options_are_validated_on_the_host():
     """The options this package adds to or honours from the reference's keyword set: chunk_size_intra -> state stride
     (mlstm_kernels/triton/chunkwise/kernel_param_heuristics.py:118-121), kernel path, head norm, state dtype."""
-    from mlstm_kernels_amd.torch.chunkwise.hip_xl_chunk import _state_stride
+    from mlstm_kernels_amd.torch.chunkwise.hip_xl_chunk import _recompute_states, _state_stride
     from mlstm_kernels_amd.torch.recurrent.hip_step import _check_state_dtype
 
+    # recompute_states_in_bw (mlstm_kernels/torch/chunkwise/triton_xl_chunk/fwbw.py:45,62): honoured, default False here
+    assert _recompute_states({}) is False and _recompute_states({"recompute_states_in_bw": None}) is False
+    assert _recompute_states({"recompute_states_in_bw": True}) is True
+    assert _recompute_states({"recompute_states_in_bw": False}) is False
+    with pytest.raises(ValueError):
+        _recompute_states({"recompute_states_in_bw": "yes"})
     assert _state_stride({}, "op") == 0                                   # library default
     assert _state_stride({"chunk_size_intra": 128}, "op") == 1
     assert _state_stride({"chunk_size_inter": 128, "chunk_size_intra": 512}, "op") == 4

@@ -651,6 +651,67 @@ def test_chunkwise_takes_16_bit_gates(dtype, siging):
         assert rel_to_scale(leaf.grad, r) <= 5e-2, name
 
 
+@pytest.mark.parametrize("kw", [
+    dict(B=2, NH=2, S=1024, DQK=256, DHV=512, seed=50),
+    dict(B=1, NH=2, S=640, DQK=128, DHV=256, seed=51, init=True, last=True),
+    dict(B=1, NH=2, S=512, DQK=64, DHV=128, seed=52, siging=True, init=True),
+    dict(B=2, NH=1, S=300, DQK=128, DHV=128, seed=53, any_s=True),
+    dict(B=1, NH=2, S=512, DQK=256, DHV=512, seed=54, dtype=torch.float16, last=True),
+])
+def test_recompute_states_in_bw_matches_kept_states(kw, kernel_variant):
+    """recompute_states_in_bw=True (the reference's saved-state policy, triton_xl_chunk/fwbw.py:45-62, bw.py:75-95): the
+    autograd function keeps only the small front part of the forward workspace and the backward runs the state scan
+    again.  Same H bit for bit; the gradients equal those of the kept-states call bit for bit on the split path when no
+    last state was returned, and to a fraction of the 16-bit rounding otherwise (a forward that returns the last state
+    carries a remainder of the scan's value operand in its late chunks, and the fused forward groups the products of a
+    chunk state differently from the scan; the recomputed states come from the plain scan).  The memory held between
+    forward and backward shrinks by the chunk states."""
+    exp_op, sig_op, *_ = _ops()
+    B, NH, S, DQK, DHV = kw["B"], kw["NH"], kw["S"], kw["DQK"], kw["DHV"]
+    siging, init, last = kw.get("siging", False), kw.get("init", False), kw.get("last", False)
+    dtype = kw.get("dtype", torch.bfloat16)
+    if dtype == torch.float16 and kernel_variant.startswith("fused"):
+        pytest.skip("the fused path multiplies bfloat16 operands only")
+    q, k, v, i, f = make_qkvif(B, NH, S, DQK, DHV, seed=kw["seed"], dtype=dtype)
+    g = torch.Generator().manual_seed(kw["seed"] + 1000)
+    dH = torch.randn(B, NH, S, DHV, generator=g).to(dtype).to(DEV)
+    c0 = (0.1 * torch.randn(B, NH, DQK, DHV, generator=g)).to(DEV) if init else None
+    n0 = (0.1 * torch.randn(B, NH, DQK, generator=g)).abs().to(DEV) if init else None
+    m0 = torch.zeros(B, NH, 1, device=DEV) if init else None
+    op = sig_op if siging else exp_op
+
+    def run(recompute):
+        leaves = [t.to(DEV).requires_grad_(True) for t in (q, k, v, i, f)]
+        c0l = c0.clone().requires_grad_(True) if init else None
+        torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated()
+        out = op(*leaves, c_initial=c0l, n_initial=n0, m_initial=m0, return_last_states=last, chunk_size=128,
+                 any_sequence_length=kw.get("any_s", False), recompute_states_in_bw=recompute)
+        H = out[0] if last else out
+        torch.cuda.synchronize()
+        held = torch.cuda.memory_allocated() - base
+        H.backward(dH)
+        grads = [t.grad for t in leaves] + ([c0l.grad] if init else [])
+        return H.detach(), grads, held
+
+    H_keep, g_keep, held_keep = run(False)
+    H_rec, g_rec, held_rec = run(True)
+    assert torch.equal(H_keep, H_rec)
+    exact = kernel_variant.startswith("split") and not last
+    for name, a, b in zip(["dQ", "dK", "dV", "dI", "dF", "dC0"], g_rec, g_keep):
+        if exact:
+            assert torch.equal(a, b), f"{name} differs from the kept-states call"
+        else:
+            # two roundings of nearly equal values to the 16-bit output format: at most one unit (2^-8 of the
+            # element) apart almost everywhere
+            assert rel_to_scale(a, b) <= 1e-2, f"{name}: {rel_to_scale(a, b):.2e} of the tensor scale"
+            assert rel_norm(a, b) <= 2e-3, f"{name}: norm error {rel_norm(a, b):.2e}"
+    stride = int(kernel_variant.split("-")[1])
+    NC = (S + 127) // 128
+    state_bytes = B * NH * ((NC + stride - 1) // stride) * DQK * DHV * 2
+    assert held_keep - held_rec >= 0.9 * state_bytes, (held_keep, held_rec, state_bytes)
+
+
 def test_chunkwise_fwbw_in_hip_graph():
     """Forward and backward of the chunkwise operator captured once in a HIP graph (workspaces from the graph's memory
     pool, no memset nodes: the library clears with fill kernels) and replayed on new data, with eager passes between
