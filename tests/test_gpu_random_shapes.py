@@ -1,5 +1,6 @@
 """Randomised parity sweep: shapes (ragged sequence lengths, head dimensions that are multiples of 64 only), both
-gates, initial states, an upstream dC_last, both chunkwise paths and every state stride, each against the fp64 oracle.  Tolerances are
+gates, initial states, an upstream dC_last, both chunkwise paths, every state stride and both saved-state policies
+(chunk states kept for the backward or recomputed in it), each against the fp64 oracle.  Tolerances are
 norm-relative (bf16 operands): H 6e-3, gradients 8e-3, final C 1e-3 of its scale, gate gradients 5e-2 of theirs."""
 import random
 
@@ -24,6 +25,7 @@ def _case(seed):
     cfg["stride"] = rnd.choice([1, 2, 3, 4, 8])
     if cfg["DQ"] not in (128, 256):
         cfg["fused"] = False   # the fused path supports these two head dimensions only
+    cfg["recompute"] = rnd.random() < 0.35
     return cfg
 
 
@@ -53,7 +55,7 @@ def test_random_shape_forward_backward(seed):
     c0l = None if c0 is None else cu(c0).requires_grad_(True)
     kw = dict(c_initial=c0l, n_initial=cu(n0), m_initial=cu(m0), return_last_states=True, chunk_size=128,
               any_sequence_length=True, kernel_path="fused" if c["fused"] else "split",
-              chunk_size_intra=128 * c["stride"])
+              chunk_size_intra=128 * c["stride"], recompute_states_in_bw=c["recompute"])
     print(f"case {c}", flush=True)
     if sig:
         H, st = mlstm_siging_chunkwise__hip_xl_chunk(*leaves, normalize=normalize, **kw)
