@@ -57,8 +57,12 @@ const char* mlstm_hip_last_error(void);
  * path: kernel selection for the value-column side of the passes (H forward, dV backward).  No counterpart in the
  * reference, whose Triton kernels are always the two-kernel form, recurrent_fw_C followed by parallel_fw_Hintra
  * (mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:20-136).
- *   MLSTM_PATH_AUTO  : the faster one for the shape as measured on MI355X (today: split for every shape)
+ *   MLSTM_PATH_AUTO  : the fastest one for the shape as measured on MI355X (stream where it applies, else split)
  *   MLSTM_PATH_SPLIT : state scan + chunk-parallel kernel over materialised chunk states
+ *   MLSTM_PATH_STREAM: the split form with the chunk-parallel kernels as persistent workgroups whose waves are split
+ *                      into producers (global memory -> LDS, several slabs in flight) and consumers (matrix
+ *                      instructions); DHQK = 256, DHHV a multiple of 256, S a multiple of 128, no head norm: other
+ *                      shapes are rejected.  Same workspaces as MLSTM_PATH_SPLIT.
  *   MLSTM_PATH_FUSED : one sequential kernel per pass, state slice resident in registers (DHQK = 128 or 256 only:
  *                      other head dimensions are rejected)
  *
@@ -75,6 +79,7 @@ const char* mlstm_hip_last_error(void);
 #define MLSTM_PATH_AUTO 0
 #define MLSTM_PATH_SPLIT 1
 #define MLSTM_PATH_FUSED 2
+#define MLSTM_PATH_STREAM 3
 
 /*
  * head_norm: optional normalisation of every row of H over its DHHV columns, fused into the epilogue of the forward

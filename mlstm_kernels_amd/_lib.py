@@ -12,7 +12,7 @@ _lib = None
 F32, BF16 = 0, 1
 F16 = 2
 GATE_EXP, GATE_SIG = 0, 1
-PATH_AUTO, PATH_SPLIT, PATH_FUSED = 0, 1, 2
+PATH_AUTO, PATH_SPLIT, PATH_FUSED, PATH_STREAM = 0, 1, 2, 3
 NORM_NONE, NORM_LAYER, NORM_RMS = 0, 1, 2
 ABI_VERSION = 6
 NOALLOC_SCRATCH_BYTES = 64 << 20  # MLSTM_NOALLOC_SCRATCH_BYTES of include/mlstm_hip.h
@@ -75,7 +75,7 @@ def get_lib() -> ctypes.CDLL:
     return _lib
 
 
-_PATH_CODES = {"auto": PATH_AUTO, "split": PATH_SPLIT, "fused": PATH_FUSED}
+_PATH_CODES = {"auto": PATH_AUTO, "split": PATH_SPLIT, "fused": PATH_FUSED, "stream": PATH_STREAM}
 _NORM_CODES = {"none": NORM_NONE, "layer": NORM_LAYER, "rms": NORM_RMS}
 
 
@@ -88,7 +88,7 @@ def norm_code(name: str) -> int:
 
 
 def path_code(name: str) -> int:
-    """'auto' / 'split' / 'fused' -> the C ABI's kernel path code."""
+    """'auto' / 'split' / 'fused' / 'stream' -> the C ABI's kernel path code."""
     try:
         return _PATH_CODES[name]
     except KeyError:

@@ -69,11 +69,21 @@ bool use_fused(int path, int DHQK, int DHHV) { return path == MLSTM_PATH_FUSED &
 constexpr int kDefaultStateStride = 2;
 int resolve_stride(int state_stride) { return state_stride == 0 ? kDefaultStateStride : state_stride; }
 const char* check_options(int path, int state_stride, int DHQK, int DHHV) {
-  if (path != MLSTM_PATH_AUTO && path != MLSTM_PATH_SPLIT && path != MLSTM_PATH_FUSED) return "unknown kernel path code";
+  if (path != MLSTM_PATH_AUTO && path != MLSTM_PATH_SPLIT && path != MLSTM_PATH_FUSED && path != MLSTM_PATH_STREAM)
+    return "unknown kernel path code";
   if (path == MLSTM_PATH_FUSED && !mlstm::fused_hv_supported(DHQK, DHHV))
     return "the fused kernel path supports DHQK = 128 or 256 only";
   if (state_stride < 0 || state_stride > mlstm::kMaxStateStride) return "state_stride must be 0 (default) or 1 .. 8";
   return nullptr;
+}
+// H / dV kernel of the split form: the streaming kernel where the path asks for it (or leaves the choice open) and the
+// shape is one it supports, otherwise the tiled kernel
+const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, hipStream_t st) {
+  if (path == MLSTM_PATH_STREAM && !mlstm::stream_hv_supported(a))
+    return "the stream kernel path supports DHQK = 256, DHHV % 256 == 0, S % 128 == 0 without head norm only";
+  if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::stream_hv_supported(a))
+    return mlstm::launch_stream_hv(a, BH, is_dv, st);
+  return mlstm::launch_par_hv(a, BH, is_dv, st);
 }
 const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {
   if (B <= 0 || NH <= 0 || S <= 0) return "B, NH and S must be positive";
@@ -305,7 +315,7 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   pa.norm_rstd = norm_rstd;
   {
     ProfileScope ps("par_h", st);
-    if (const char* e = mlstm::launch_par_hv(pa, BH, /*is_dv=*/false, st)) return fail(e);
+    if (const char* e = launch_hv(path, pa, BH, /*is_dv=*/false, st)) return fail(e);
   }
   return check_launch("par_hv forward");
 }
@@ -469,7 +479,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
     pv.f16 = f16;
     {
       ProfileScope ps("par_dv", st);
-      if (const char* e = mlstm::launch_par_hv(pv, BH, /*is_dv=*/true, st)) return fail(e);
+      if (const char* e = launch_hv(path, pv, BH, /*is_dv=*/true, st)) return fail(e);
     }
     if (check_launch("par_hv dV")) return 1;
   }

@@ -120,6 +120,9 @@ const char* launch_gates(const void* i, const void* f, const float* m0, const Ga
 const char* launch_scan(const ScanArgs& a, int BH, bool hilo, hipStream_t stream);
 const char* launch_par_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 bool par_hv_head_norm_supported(int DHHV);
+// streaming (persistent, producer / consumer waves) form of the same two kernels for the shapes it supports
+bool stream_hv_supported(const ParHvArgs& a);
+const char* launch_stream_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 const char* launch_head_norm_bw(const HeadNormBwArgs& a, hipStream_t stream);
 bool fused_hv_supported(int DHQK, int DHHV);
 const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream);

@@ -1,0 +1,610 @@
+// Streaming form of the chunk-parallel kernels whose output tile spans value columns (forward output H, gradient dV):
+// the same arithmetic as par_hv.hip (see there for the formulas and the state-stride algebra), organised for a step
+// whose binding resource is HBM bandwidth rather than the matrix pipes.
+//
+//   * One PERSISTENT workgroup per CU (sixteen waves) walks its share of the work items; an item is one chunk of 128
+//     positions x 256 value columns of one (batch, head).
+//   * The waves have two roles.  Eight PRODUCER waves do nothing but move data: every operand of every item -- the 128
+//     resident rows (Q forward, K for dV), the kept state as ready-made operand fragments, the rows of the source
+//     chunks for the scores and for the output product -- is cut into slabs of 32 KB, and the producers always have two
+//     slabs (64 KB per CU) on their way from memory in registers, across item boundaries, so the memory pipe does not
+//     drain while an item starts up or is written out.  Eight CONSUMER waves read operand fragments from LDS, multiply
+//     (sixteen matrix instructions per wave and slab), gate the score blocks and write the output; they never wait
+//     for global memory.
+//   * The two roles meet at ONE barrier per slab: after barrier g the consumers work on slab g while the producers
+//     write slab g+1 into the other ring slot and request slab g+3.  Both roles walk the same item list with the same
+//     number of steps per item (6 + 4 per source chunk), so they pass the same number of barriers by construction.
+//   * The output of an item is written while the resident rows of the next item arrive (those two steps carry no
+//     operand the consumers could use), transposed through the score block, which is idle then.
+//
+// Step sequence of an item (s source chunks, the own chunk last):
+//   2 x resident rows (64 rows each, written straight into their LDS tile)
+//   4 x state slab: 4 contraction steps x 8 fragment blocks of 32 value columns
+//   per source chunk, per half of 64 source positions: 1 slab of 64 rows x DHQK (scores, gated into the score block
+//   in the same step), 1 slab of 64 rows x 256 value columns (output product)
+// Every phase has an even number of steps, so the register set and the ring slot of a step are known at compile time.
+// Supported: DHQK = 256, DHHV a multiple of 256, S a multiple of 128, no head norm; everything else runs par_hv.hip.
+#include "common.h"
+#include "kernels.h"
+
+namespace mlstm {
+namespace {
+
+struct HvItem {
+  int bh, c, ch;               // (batch * head), chunk, group of 256 value columns
+  int slot;                    // kept boundary state the chunk uses
+  int sc_first, sc_step, nsc;  // source chunks: sc_first, sc_first + sc_step, ... (nsc of them, the own chunk last)
+};
+
+// Work item of workgroup `vid` in round `round`.  Consecutive workgroups take consecutive items (the column groups of
+// a chunk, then the next chunk: they share rows and kept states through the L2 of their XCD); the assignment rotates
+// by one chunk per round so that a workgroup does not always get the chunks with the same number of source chunks.
+template <bool IS_DV>
+__device__ __forceinline__ bool hv_decode(HvItem& it, int round, int vid, int G, int n_items, int NC, int NCH, int stride) {
+  const int rot = (vid + round * NCH) % G;
+  const long long idx = (long long)round * G + rot;
+  if (idx >= n_items) return false;
+  const int i = (int)idx;
+  it.ch = i % NCH;
+  const int rest = i / NCH;
+  it.c = rest % NC;
+  it.bh = rest / NC;
+  it.slot = it.c / stride;
+  if (IS_DV) {
+    const int hi = min(it.slot * stride + stride - 1, NC - 1);
+    it.sc_first = hi;
+    it.sc_step = -1;
+    it.nsc = hi - it.c + 1;
+  } else {
+    it.sc_first = it.slot * stride;
+    it.sc_step = 1;
+    it.nsc = it.c - it.sc_first + 1;
+  }
+  return true;
+}
+
+}  // namespace
+
+#ifdef HV_EXP_TIMING
+__device__ unsigned long long g_hv_dbg[32];
+#define HV_SYNC()                                                     \
+  {                                                                   \
+    const unsigned long long t0_ = __builtin_amdgcn_s_memrealtime();  \
+    __syncthreads();                                                  \
+    const unsigned long long t1_ = __builtin_amdgcn_s_memrealtime();  \
+    dbg_wait += t1_ - t0_;                                            \
+    dbg_n += 1;                                                       \
+  }
+#define HV_PHASE(k)
+#define HV_TB(k) unsigned long long treg_##k = 0; if ((k) == HV_T_REGION) treg_##k = __builtin_amdgcn_s_memrealtime();
+#define HV_TE(k) if ((k) == HV_T_REGION) { dbg_reg += __builtin_amdgcn_s_memrealtime() - treg_##k; dbg_regn += 1; }
+#else
+#define HV_SYNC() __syncthreads()
+#define HV_PHASE(k)
+#define HV_TB(k)
+#define HV_TE(k)
+#endif
+template <bool IS_DV, bool F16>
+__global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_items, int n_rounds) {
+  constexpr int DHQK = 256;
+  constexpr int QS = DHQK + 8;   // resident rows [128][DHQK] and score-operand slabs [64][DHQK], fragment order
+  constexpr int VS = 256 + 16;   // value-operand slab: 64 rows x 256 value columns, row-major
+  constexpr int PSS = 64 + 8;    // gated score block P[n][o]: 128 positions x 64 source positions
+  constexpr int SLOT = 64 * VS;  // elements per ring slot (the largest slab kind)
+  constexpr int ND = DHQK / 16;
+  static_assert(64 * QS <= SLOT && 16384 <= SLOT, "every slab kind fits a ring slot");
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  uint16_t* const Ns = (uint16_t*)smem_raw;
+  uint16_t* const Ps = Ns + 128 * QS;
+  uint16_t* const Ring = Ps + 128 * PSS;
+  float* const rows = (float*)(Ring + 2 * SLOT);  // [4][128] partial row sums of the own chunk's scores (forward)
+  float* const inv = rows + 4 * 128;              // [128] forward: 1 / (row normaliser + eps)
+  float* const nperm = inv + 128;                 // [DHQK] forward: n before the chunk, fragment order
+  float* const ovec = nperm + DHQK;               // [64] gate vector of the source half: w_j (forward) / u_t (dV)
+  float* const orho = ovec + 64;                  // [64] dV: rho_t of the source half
+  constexpr uint32_t kRingOff = (128 * QS + 128 * PSS) * 2;
+
+#ifdef HV_EXP_TIMING
+  unsigned long long dbg_wait = 0, dbg_n = 0;
+  unsigned long long dbg_reg = 0, dbg_regn = 0;
+  const unsigned long long dbg_start = __builtin_amdgcn_s_memrealtime();
+#endif
+  const int lane = threadIdx.x & 63;
+  const int wave_all = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int G = gridDim.x;
+  int vid = blockIdx.x;
+  if (G % 8 == 0) vid = (vid % 8) * (G / 8) + vid / 8;  // consecutive ids share an XCD (and its L2)
+  const int NC = a.NC, S = a.S, DHHV = a.DHHV, NCH = DHHV / 256, stride = a.stride;
+  const size_t Sp = (size_t)NC * kChunk;
+  const int NCS = (NC + stride - 1) / stride;
+
+  if (wave_all >= 8) {
+    // =========================================================================================== producer waves
+    // Load step L (counted over all items of this workgroup) uses register set L & 1.  Handling it means: pass barrier
+    // L - 3 (the consumers are done with slab L - 4, whose ring slot slab L - 2 goes into), write slab L - 2 from the
+    // register set to LDS, request slab L into the set.  The destination in LDS travels with the data: byte offset of
+    // the thread's first piece | slab kind << 20 (0 fragment-order rows, 1 state fragments, 3 value rows) | gate-vector
+    // flag << 22; the thread's other three pieces lie a fixed distance apart.
+    const int p = (wave_all - 8) * 64 + lane;  // 0 .. 511: every thread moves four 16-byte pieces of every slab
+    const char* const Xn_b = (const char*)(IS_DV ? a.K : a.Q);
+    const char* const Xo_b = (const char*)(IS_DV ? a.Q : a.K);
+    const char* const Xw_b = (const char*)(IS_DV ? a.dH : a.V);
+    const char* const St_b = (const char*)a.states;
+    const float* const ov_src = IS_DV ? a.g.u : a.g.w;
+    const float* const rho_src = (IS_DV && a.use_nrow) ? a.nrow : ov_src;
+    uint4 fd[2][4];
+    uint32_t fw[2];
+    float fa[2][2];
+    int L = 0;
+#define HV_STORE(E)                                                                                                  \
+  {                                                                                                                  \
+    const uint32_t w_ = fw[E];                                                                                       \
+    const uint32_t kind_ = (uint32_t)__builtin_amdgcn_readfirstlane((int)((w_ >> 20) & 3));                          \
+    const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
+    const uint32_t half_ = kind_ == 0 ? 16u : 8u;                                                                    \
+    const uint32_t step_ = kind_ == 0 ? 16 * QS * 2 : (kind_ == 1 ? 8192 : 16 * VS * 2);                             \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                               \
+      *(uint2*)(smem_raw + d0_ + i_ * step_) = make_uint2(fd[E][i_].x, fd[E][i_].y);                                 \
+      *(uint2*)(smem_raw + d0_ + i_ * step_ + half_) = make_uint2(fd[E][i_].z, fd[E][i_].w);                         \
+    }                                                                                                                \
+    if (__builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 64) {                                           \
+      ovec[p] = fa[E][0];                                                                                            \
+      if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa[E][1] + a.eps) : 1.f;                                              \
+    }                                                                                                                \
+  }
+    // base_: (batch, head) base of the operand; g0_: byte offset of the thread's first piece, gs_: distance between
+    // its pieces; gi_: index of the gate-vector entry that rides along (stored only with the flag set; the other
+    // slabs request an entry all the same so that every step issues the same loads)
+#define HV_PROC(E, base_, g0_, gs_, dstw_, gi_)                                                                      \
+  {                                                                                                                  \
+    if (L >= 3) HV_SYNC();                                                                                     \
+    HV_TB(6) if (L >= 2) HV_STORE(E) HV_TE(6)                                                                         \
+    HV_TB(7) HV_EXP_LOADS(E, base_, g0_, gs_, gi_) HV_TE(7)                                                           \
+    fw[E] = (dstw_);                                                                                                 \
+    ++L;                                                                                                             \
+  }
+#ifdef HV_EXP_NOLOAD
+#define HV_EXP_LOADS(E, base_, g0_, gs_, gi_)                                                                        \
+  {                                                                                                                  \
+    fa[E][0] = (float)(g0_); fa[E][1] = 1.f;                                                                         \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd[E][i_] = make_uint4((g0_) + i_ * (gs_), 0, 0, 0);            \
+    (void)(base_); (void)(gi_);                                                                                      \
+  }
+#else
+#define HV_EXP_LOADS(E, base_, g0_, gs_, gi_)                                                                        \
+  {                                                                                                                  \
+    fa[E][0] = ov_src[gi_];                                                                                          \
+    fa[E][1] = rho_src[gi_];                                                                                         \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd[E][i_] = *(const uint4*)((base_) + ((g0_) + i_ * (gs_)));    \
+  }
+#endif
+    HvItem it;
+    for (int rd = 0; rd < n_rounds; ++rd) {
+      if (!hv_decode<IS_DV>(it, rd, vid, G, n_items, NC, NCH, stride)) continue;
+      const uint32_t pl = (uint32_t)opaque(p);
+      const uint32_t row = pl >> 5, pc = pl & 31;  // rows of 512 bytes: 32 pieces per row, 16 rows per sweep
+      const size_t gown = (size_t)it.bh * Sp + (size_t)it.c * kChunk + (pl & 63);
+      // fragment-order destination of piece pc inside a row (see store_perm16)
+      const uint32_t permo = (pc >> 1) * 32 + 8 * (pc & 1);
+      {
+        // ---- resident rows
+        const char* const base = Xn_b + (size_t)it.bh * S * DHQK * 2;
+        const uint32_t g0 = ((uint32_t)(it.c * kChunk) + row) * (DHQK * 2) + pc * 16;
+        const uint32_t d0 = row * (QS * 2) + permo;
+        HV_PROC(0, base, g0, 16 * DHQK * 2, d0, gown)
+        HV_PROC(1, base, g0 + 64 * DHQK * 2, 16 * DHQK * 2, d0 + 64 * QS * 2, gown)
+      }
+      {
+        // ---- state fragments: slab si holds contraction steps 4 si .. 4 si + 3 of the eight 32-column blocks
+        const char* const base = St_b + ((size_t)it.bh * NCS + it.slot) * (size_t)(DHHV / 32) * ND * 1024;
+        const uint32_t wbl = pl >> 8, dsl = (pl >> 6) & 3;
+        const uint32_t g0 = (((uint32_t)it.ch * 8 + wbl) * ND + dsl) * 1024 + (pl & 63) * 16;
+        for (int si = 0; si < 4; si += 2) {
+          HV_PROC(0, base, g0 + si * 4096, 2 * ND * 1024, (kRingOff + pl * 16) | (1u << 20), gown)
+          HV_PROC(1, base, g0 + (si + 1) * 4096, 2 * ND * 1024, (kRingOff + SLOT * 2 + pl * 16) | (1u << 20), gown)
+        }
+      }
+      {
+        const char* const kbase = Xo_b + (size_t)it.bh * S * DHQK * 2;
+        const char* const vbase = Xw_b + (size_t)it.bh * S * DHHV * 2;
+        const uint32_t kd0 = kRingOff + row * (QS * 2) + permo;
+        const uint32_t vd0 = (kRingOff + SLOT * 2 + row * (VS * 2) + pc * 16) | (3u << 20);
+        for (int sci = 0; sci < it.nsc; ++sci) {
+          const int sc = it.sc_first + sci * it.sc_step;
+          for (int kh = 0; kh < 2; ++kh) {
+            const uint32_t t0 = (uint32_t)(sc * kChunk + 64 * kh) + row;
+            const size_t gi = (size_t)it.bh * Sp + (size_t)sc * kChunk + 64 * kh + (pl & 63);
+            HV_PROC(0, kbase, t0 * (DHQK * 2) + pc * 16, 16 * DHQK * 2, kd0 | (1u << 22), gi)
+            HV_PROC(1, vbase, t0 * (uint32_t)(DHHV * 2) + (uint32_t)it.ch * 512 + pc * 16, 16 * (uint32_t)DHHV * 2, vd0, gown)
+          }
+        }
+      }
+    }
+    // ---- drain: the last two slabs go to LDS, then the barriers of the consumers' last steps and of the final epilogue
+    if (L > 0) {
+      if (L >= 3) HV_SYNC();
+      HV_STORE(0)
+      HV_SYNC();
+      HV_STORE(1)
+      HV_SYNC();
+      HV_SYNC();
+      HV_SYNC();
+    }
+#undef HV_PROC
+#undef HV_EXP_LOADS
+#undef HV_STORE
+  } else {
+    // =========================================================================================== consumer waves
+#ifdef HV_EXP_NOMFMA
+#define HV_MFMA(C_, A_, B_) { (C_)[0] += __uint_as_float((A_).w[0] ^ (B_).w[0]); }
+#else
+#define HV_MFMA(C_, A_, B_) mfma32<F16>(C_, A_, B_)
+#endif
+#ifdef HV_EXP_PRIO
+    __builtin_amdgcn_s_setprio(HV_EXP_PRIO);
+#endif
+    const int wave = wave_all;
+    const int tid = wave * 64 + lane;
+    const int pi = wave & 1, ci = wave >> 1;  // output role: positions 64 pi .., value columns 64 ci .. of the item
+    const int pb = wave & 3, kb = wave >> 2;  // score role: position block pb, source block kb of a 64-position half
+    f32x16 acc[2][2], sacc;
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
+    HvItem it, prev;
+    prev = HvItem{0, 0, 0, 0, 0, 1, 1};
+    bool have_prev = false;
+    // The accumulators are only ever touched in straight-line code between barriers: no matrix instruction sits under
+    // a condition (dead score blocks of the own chunk are multiplied and masked to zero by the gating), so the
+    // compiler keeps every accumulator in one place.  The epilogue is a macro with a literal position block:
+    // (normalise,) round, transpose 32 positions x 64 columns through a private part of the idle score block,
+    // coalesced non-temporal stores.
+#define HV_EPILOGUE(NB)                                                                                              \
+  {                                                                                                                  \
+    const int le = opaque(lane);                                                                                     \
+    const int r = le & 31, h = le >> 5;                                                                              \
+    constexpr int SR = 64 + 8; /* staging row: 64 value columns */                                                   \
+    uint16_t* const stg = Ps + (wave & 3) * (32 * SR);                                                               \
+    const float iv = IS_DV ? 1.f : inv[64 * pi + 32 * NB + r];                                                       \
+    _Pragma("unroll") for (int mb = 0; mb < 2; ++mb) _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {              \
+      *(uint2*)(stg + r * SR + 32 * mb + 8 * g4 + 4 * h) =                                                           \
+          make_uint2(pack2<F16>(acc[mb][NB][4 * g4 + 0] * iv, acc[mb][NB][4 * g4 + 1] * iv),                         \
+                     pack2<F16>(acc[mb][NB][4 * g4 + 2] * iv, acc[mb][NB][4 * g4 + 3] * iv));                        \
+    }                                                                                                                \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                           \
+    __builtin_amdgcn_wave_barrier();                                                                                 \
+    uint16_t* const Og = a.Out + ((size_t)prev.bh * S + (size_t)prev.c * kChunk + 64 * pi + 32 * NB) * DHHV +        \
+                         prev.ch * 256 + 64 * ci;                                                                    \
+    _Pragma("unroll") for (int k = 0; k < 4; ++k) {                                                                  \
+      const int row = (le >> 3) + 8 * k, pc = le & 7;                                                                \
+      __builtin_nontemporal_store(*(const u32x4*)(stg + row * SR + pc * 8), (u32x4*)(Og + (size_t)row * DHHV + pc * 8)); \
+    }                                                                                                                \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                           \
+    __builtin_amdgcn_wave_barrier();                                                                                 \
+  }
+    for (int rd = 0; rd < n_rounds; ++rd) {
+      if (!hv_decode<IS_DV>(it, rd, vid, G, n_items, NC, NCH, stride)) continue;
+      const int bh = it.bh, c = it.c;
+      const size_t hofs = (size_t)bh * Sp, gofs = hofs + (size_t)c * kChunk;
+      const float* graw = a.g.graw + (size_t)bh * NC;
+      const float* mst = a.g.mstates + (size_t)bh * (NC + 1);
+      // ---- two steps while the resident rows arrive: the previous item's output leaves (waves 0..3 in the first
+      // step, 4..7 in the second: the staging area holds four tiles), the per-item vectors are requested
+      float csr[2], nv, cs0r = 0.f, mcr = 0.f, np0 = 0.f, np1 = 0.f, np2 = 0.f, qn = 0.f;
+      HV_SYNC();
+      HV_TB(5)
+      if (have_prev && wave < 4) {
+        HV_EPILOGUE(0)
+        HV_EPILOGUE(1)
+      }
+      {
+        const int r = opaque(lane) & 31;
+        float gsum = 0.f, xs = 1.f;
+        if (IS_DV) {
+          const int hi = it.sc_first;
+          for (int x = c + 1; x <= hi; ++x) gsum += graw[x];
+          if (hi > c) xs = __expf(gsum + mst[c + 1] - mst[hi + 1]);
+        } else {
+          const int lo = it.sc_first;
+          for (int x = lo; x < c; ++x) gsum += graw[x];
+          if (lo < c) xs = __expf(gsum + mst[lo] - mst[c]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          const size_t gi = gofs + 64 * pi + 32 * nb + r;
+          csr[nb] = (IS_DV ? a.g.abar[gi] : a.g.bbar[gi] * a.qk_scale) * xs;
+        }
+        nv = (IS_DV ? a.g.w : a.g.u)[gofs + 32 * pb + r];
+        if (!IS_DV) {
+          const int t = opaque(tid) >> 2;
+          cs0r = a.g.bbar[gofs + t] * a.qk_scale;
+          mcr = a.g.mcomb[gofs + t];
+          if (tid < DHQK) {
+            // the scan hands n over as three partial vectors per chunk (their sum carries the full fp32 precision)
+            const float* np3 = a.nstates + ((size_t)bh * NC + c) * 3 * DHQK + tid;
+            np0 = np3[0];
+            np1 = np3[DHQK];
+            np2 = np3[2 * DHQK];
+          }
+        }
+      }
+      HV_TE(5)
+      HV_SYNC();
+      if (have_prev && wave >= 4) {
+        HV_EPILOGUE(0)
+        HV_EPILOGUE(1)
+      }
+      // ---- inter-chunk product: Out^T = State^T Xn^T, four contraction steps per slab
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
+      // (the operand fragments that do not depend on the incoming slab -- resident rows -- are requested before the
+      // barrier of a step, while the wave would otherwise only wait)
+      Frag Bpre[2];
+      {
+        const int le = opaque(lane);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) Bpre[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + (le & 31)) * QS + 8 * (le >> 5));
+      }
+#pragma unroll
+      for (int si = 0; si < 4; ++si) {
+        HV_SYNC();
+        HV_PHASE(1)
+        if (!IS_DV) {
+          if (si == 0 && tid < DHQK) nperm[perm16(tid)] = (np0 + np1) + np2;
+          if (si == 1) {
+            // forward: q_t . n_prev for the denominators (four threads per position), while the resident rows are
+            // all there -- the next item's rows start to arrive during this item's last step
+            const int td = opaque(tid);
+            const int t = td >> 2, part = td & 3;
+            const uint16_t* qrow = Ns + t * QS + part * (DHQK / 4);
+            const float* np = nperm + part * (DHQK / 4);
+            float dot = 0.f;
+#pragma unroll 2
+            for (int d = 0; d < DHQK / 4; d += 8) {
+              const uint4 qv = *(const uint4*)(qrow + d);
+              const float4 na = *(const float4*)(np + d), nb4 = *(const float4*)(np + d + 4);
+              dot += lo2<F16>(qv.x) * na.x + hi2<F16>(qv.x) * na.y + lo2<F16>(qv.y) * na.z + hi2<F16>(qv.y) * na.w;
+              dot += lo2<F16>(qv.z) * nb4.x + hi2<F16>(qv.z) * nb4.y + lo2<F16>(qv.w) * nb4.z + hi2<F16>(qv.w) * nb4.w;
+            }
+            dot += __shfl_xor(dot, 1);
+            dot += __shfl_xor(dot, 2);
+            qn = dot;
+          }
+        }
+        HV_TB(1)
+        const int le = opaque(lane);
+        const int r = le & 31, h = le >> 5;
+        const uint16_t* const slab = Ring + (si & 1) * SLOT;
+#pragma unroll
+        for (int dsl = 0; dsl < 4; ++dsl) {
+          Frag A[2], B[2];
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb) A[mb].u = *(const uint4*)(slab + ((2 * ci + mb) * 4 + dsl) * 512 + le * 8);
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) {
+            if (dsl == 0) B[nb] = Bpre[nb];
+            else B[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + r) * QS + 16 * (4 * si + dsl) + 8 * h);
+          }
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) HV_MFMA(acc[mb][nb], A[mb], B[nb]);
+        }
+        if (si < 3) {
+#pragma unroll
+          for (int nb = 0; nb < 2; ++nb) Bpre[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + r) * QS + 16 * (4 * si + 4) + 8 * h);
+        }
+        HV_TE(1)
+      }
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= csr[nb];
+
+      // ---- source chunks (the own chunk last), 64 source positions at a time
+      for (int sci = 0; sci < it.nsc; ++sci) {
+        const int sc = it.sc_first + sci * it.sc_step;
+        const bool own = sc == c;
+        float gs = 0.f;  // decay between the source chunk and this chunk
+        for (int x = (IS_DV ? c : sc); x < (IS_DV ? sc : c); ++x) gs += graw[x];
+        for (int kh = 0; kh < 2; ++kh) {
+          // scores of position block pb against source block kb of this half
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+          Frag Bk[4];
+          {
+            const int le = opaque(lane);
+#pragma unroll
+            for (int ds = 0; ds < 4; ++ds) Bk[ds].u = *(const uint4*)(Ns + (32 * pb + (le & 31)) * QS + 16 * ds + 8 * (le >> 5));
+          }
+          HV_SYNC();
+          HV_PHASE(2)
+          {
+            HV_TB(2)
+            const int le = opaque(lane);
+            const int r = le & 31, h = le >> 5;
+            const uint16_t* const slab = Ring;
+#pragma unroll
+            for (int ds = 0; ds < ND; ++ds) {
+              Frag A, B;
+              A.u = *(const uint4*)(slab + (32 * kb + r) * QS + 16 * ds + 8 * h);
+              if (ds < 4) B = Bk[ds];
+              else B.u = *(const uint4*)(Ns + (32 * pb + r) * QS + 16 * ds + 8 * h);
+              HV_MFMA(sacc, A, B);
+            }
+            HV_TE(2)
+            HV_TB(3)
+            // gate, mask, round and write P as Ps[n][o]; forward: fp32 row sums over the own chunk's positions
+            const int n = 32 * pb + r;  // position inside the chunk
+            const float un = nv + (IS_DV ? -gs : gs);
+            float rsum = 0.f;
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+              const int ol = 32 * kb + 8 * g4 + 4 * h;  // source position inside the half
+              const float4 xo = *(const float4*)(ovec + ol);
+              const float xov[4] = {xo.x, xo.y, xo.z, xo.w};
+              float rho[4] = {1.f, 1.f, 1.f, 1.f};
+              if (IS_DV) {
+                const float4 rr = *(const float4*)(orho + ol);
+                rho[0] = rr.x; rho[1] = rr.y; rho[2] = rr.z; rho[3] = rr.w;
+              }
+              float pv[4];
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int o = 64 * kh + ol + q;
+                const float ex = IS_DV ? (xov[q] - un) : (un - xov[q]);
+                const bool keep = !own || (IS_DV ? (n <= o) : (o <= n));
+                const float val = sacc[4 * g4 + q] * a.qk_scale * __expf(ex) * rho[q];
+                pv[q] = keep ? val : 0.f;
+                rsum += pv[q];
+              }
+              *(uint2*)(Ps + n * PSS + ol) = make_uint2(pack2<F16>(pv[0], pv[1]), pack2<F16>(pv[2], pv[3]));
+            }
+            if (!IS_DV && own) {
+              const float tot = rsum + __shfl_xor(rsum, 32);
+              if (h == 0) rows[(2 * kh + kb) * 128 + n] = tot;  // blocks above the diagonal publish zero
+            }
+            HV_TE(3)
+          }
+          // Out^T += Xw^T P over the 64 source positions of the half
+          HV_SYNC();
+          HV_PHASE(3)
+          {
+            const int le = opaque(lane);
+            const int r = le & 31, h = le >> 5;
+            const int q16 = (le >> 4) & 1, i16 = le & 15;
+            const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
+            HV_TB(4)
+            const uint16_t* const slab = Ring + SLOT;
+#pragma unroll
+            for (int k16 = 0; k16 < 4; ++k16) {
+              Frag A[2], B[2];
+#pragma unroll
+              for (int mb = 0; mb < 2; ++mb) {
+                const uint16_t* pp = slab + (16 * k16 + krow) * VS + (64 * ci + 32 * mb + ncol);
+                A[mb].d[0] = lds_read_tr16(pp);
+                A[mb].d[1] = lds_read_tr16(pp + 4 * VS);
+              }
+#pragma unroll
+              for (int nb = 0; nb < 2; ++nb)
+                B[nb].u = *(const uint4*)(Ps + (64 * pi + 32 * nb + r) * PSS + 16 * k16 + 8 * h);
+#pragma unroll
+              for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) HV_MFMA(acc[mb][nb], A[mb], B[nb]);
+            }
+            HV_TE(4)
+            // ---- forward: denominators, once all row sums of the own chunk are there (it is the last source chunk)
+            if (!IS_DV && own && kh == 1) {
+              const int td = opaque(tid);
+              const int t = td >> 2;
+              if ((td & 3) == 0) {
+                float nmax = 1.f, iv = 1.f;
+                if (a.use_nrow) {
+                  float den = cs0r * qn;
+#pragma unroll
+                  for (int b4 = 0; b4 < 4; ++b4) den += rows[b4 * 128 + t];
+                  const float floor_v = a.sig_gate ? 1.f : __expf(-mcr);
+                  nmax = fmaxf(fabsf(den), floor_v);
+                  iv = 1.f / (nmax + a.eps);
+                }
+                inv[t] = iv;
+                if (it.ch == 0) {
+                  a.nrow_out[gofs + t] = nmax;
+                  const size_t tg = (size_t)bh * S + (size_t)c * kChunk + t;
+                  if (a.n_out != nullptr) a.n_out[tg] = nmax;
+                  if (a.m_out != nullptr) a.m_out[tg] = mcr;
+                }
+              }
+            }
+          }
+        }
+      }
+      prev = it;
+      have_prev = true;
+    }
+    if (have_prev) {
+      HV_SYNC();
+      if (wave < 4) {
+        HV_EPILOGUE(0)
+        HV_EPILOGUE(1)
+      }
+      HV_SYNC();
+      if (wave >= 4) {
+        HV_EPILOGUE(0)
+        HV_EPILOGUE(1)
+      }
+    }
+#undef HV_EPILOGUE
+#undef HV_MFMA
+  }
+#ifdef HV_EXP_TIMING
+  if (blockIdx.x == 0 && lane == 0 && (wave_all == 0 || wave_all == 8)) {
+    const int o = (wave_all == 8 ? 8 : 0) + (IS_DV ? 16 : 0);
+    g_hv_dbg[o] = dbg_wait;
+    g_hv_dbg[o + 1] = dbg_n;
+    g_hv_dbg[o + 2] = __builtin_amdgcn_s_memrealtime() - dbg_start;
+    g_hv_dbg[o + 4] = dbg_reg;
+    g_hv_dbg[o + 5] = dbg_regn;
+  }
+#endif
+}
+
+bool stream_hv_supported(const ParHvArgs& a) {
+  return a.DHQK == 256 && a.DHHV % 256 == 0 && a.S % kChunk == 0 && a.head_norm == 0;
+}
+
+namespace {
+int device_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <bool IS_DV, bool F16>
+const char* launch_stream_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
+  constexpr int QS = 256 + 8, PSS = 72, SLOT = 64 * 272;
+  const size_t smem = (size_t)(128 * QS + 128 * PSS + 2 * SLOT) * 2 + (size_t)(4 * 128 + 128 + 256 + 64 + 64) * 4;
+  const long long n_items = (long long)BH * a.NC * (a.DHHV / 256);
+  if (n_items >= (1ll << 31)) return "stream_hv: too many work items";
+  if ((size_t)a.S * (size_t)a.DHHV * 2 >= ((size_t)1 << 32)) return "stream_hv: one (batch, head) slab of an input exceeds 4 GiB";
+  const int cus = device_cu_count();
+  if (cus <= 0) return "stream_hv: cannot read the number of compute units";
+  int G = (int)(n_items < cus ? n_items : cus);
+  if (G >= 8) G -= G % 8;
+  const int n_rounds = (int)((n_items + G - 1) / G);
+  if (hipFuncSetAttribute((const void*)stream_hv_kernel<IS_DV, F16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
+      hipSuccess)
+    return "stream_hv: cannot raise the dynamic LDS limit";
+  hipLaunchKernelGGL((stream_hv_kernel<IS_DV, F16>), dim3(G), dim3(1024), smem, stream, a, (int)n_items, n_rounds);
+  return nullptr;
+}
+}  // namespace
+
+const char* launch_stream_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
+  if (!stream_hv_supported(a)) return "stream_hv: unsupported shape (needs DHQK = 256, DHHV % 256 == 0, S % 128 == 0, no head norm)";
+  if (a.stride < 1 || a.stride > kMaxStateStride) return "stream_hv: state stride out of range";
+  if (is_dv) return a.f16 ? launch_stream_hv_t<true, true>(a, BH, stream) : launch_stream_hv_t<true, false>(a, BH, stream);
+  return a.f16 ? launch_stream_hv_t<false, true>(a, BH, stream) : launch_stream_hv_t<false, false>(a, BH, stream);
+}
+
+}  // namespace mlstm
+
+#ifdef HV_EXP_TIMING
+extern "C" int mlstm_debug_read(unsigned long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(mlstm::g_hv_dbg), sizeof(unsigned long long) * 32);
+}
+#endif
