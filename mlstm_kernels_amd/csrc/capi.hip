@@ -80,7 +80,7 @@ const char* check_options(int path, int state_stride, int DHQK, int DHHV) {
 // shape is one it supports, otherwise the tiled kernel
 const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, hipStream_t st) {
   if (path == MLSTM_PATH_STREAM && !mlstm::stream_hv_supported(a))
-    return "the stream kernel path supports DHQK = 256, DHHV % 256 == 0, S % 128 == 0 without head norm only";
+    return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 without head norm only";
   if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::stream_hv_supported(a))
     return mlstm::launch_stream_hv(a, BH, is_dv, st);
   return mlstm::launch_par_hv(a, BH, is_dv, st);

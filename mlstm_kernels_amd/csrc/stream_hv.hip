@@ -1,29 +1,32 @@
 // Streaming form of the chunk-parallel kernels whose output tile spans value columns (forward output H, gradient dV):
-// the same arithmetic as par_hv.hip (see there for the formulas and the state-stride algebra), organised for a step
-// whose binding resource is HBM bandwidth rather than the matrix pipes.
+// the same arithmetic as par_hv.hip (see there for the formulas and the state-stride algebra), organised around the
+// two resources that bind it on this chip: HBM bandwidth and the LDS read port of a CU (about 128 bytes per clock;
+// every matrix instruction fed from LDS costs 1 KB of it at a 2 x 2 register blocking).
 //
-//   * One PERSISTENT workgroup per CU (sixteen waves) walks its share of the work items; an item is one chunk of 128
-//     positions x 256 value columns of one (batch, head).
-//   * The waves have two roles.  Eight PRODUCER waves do nothing but move data: every operand of every item -- the 128
+//   * One PERSISTENT workgroup per CU (twelve waves) walks its share of the work items; an item is one chunk of 128
+//     positions x 512 value columns of one (batch, head), so the gated score blocks of a chunk are computed once.
+//   * The waves have two roles.  Four PRODUCER waves do nothing but move data: every operand of every item -- the 128
 //     resident rows (Q forward, K for dV), the kept state as ready-made operand fragments, the rows of the source
 //     chunks for the scores and for the output product -- is cut into slabs of 32 KB, and the producers always have two
 //     slabs (64 KB per CU) on their way from memory in registers, across item boundaries, so the memory pipe does not
-//     drain while an item starts up or is written out.  Eight CONSUMER waves read operand fragments from LDS, multiply
-//     (sixteen matrix instructions per wave and slab), gate the score blocks and write the output; they never wait
-//     for global memory.
+//     drain while an item starts up or is written out.  Eight CONSUMER waves own 64 positions x 128 columns each (128
+//     accumulator registers: three waves per SIMD leave 168 registers a wave), read operand fragments from LDS (six
+//     fragments feed eight matrix instructions), gate the score blocks and write the output; they never wait for
+//     global memory.
 //   * The two roles meet at ONE barrier per slab: after barrier g the consumers work on slab g while the producers
 //     write slab g+1 into the other ring slot and request slab g+3.  Both roles walk the same item list with the same
-//     number of steps per item (6 + 4 per source chunk), so they pass the same number of barriers by construction.
+//     number of steps per item (10 + 6 per source chunk), so they pass the same number of barriers by construction.
 //   * The output of an item is written while the resident rows of the next item arrive (those two steps carry no
-//     operand the consumers could use), transposed through the score block, which is idle then.
+//     operand the consumers could use), transposed through the ring slots and the score block, which are idle then.
 //
 // Step sequence of an item (s source chunks, the own chunk last):
 //   2 x resident rows (64 rows each, written straight into their LDS tile)
-//   4 x state slab: 4 contraction steps x 8 fragment blocks of 32 value columns
+//   8 x state slab: 2 contraction steps x 16 fragment blocks of 32 value columns
 //   per source chunk, per half of 64 source positions: 1 slab of 64 rows x DHQK (scores, gated into the score block
-//   in the same step), 1 slab of 64 rows x 256 value columns (output product)
-// Every phase has an even number of steps, so the register set and the ring slot of a step are known at compile time.
-// Supported: DHQK = 256, DHHV a multiple of 256, S a multiple of 128, no head norm; everything else runs par_hv.hip.
+//   in the same step), 2 slabs of 32 rows x 512 value columns (output product)
+// Register set and ring slot alternate from step to step and every source chunk has an even number of steps, so both
+// are compile-time constants everywhere.
+// Supported: DHQK = 256, DHHV a multiple of 512, S a multiple of 128, no head norm; everything else runs par_hv.hip.
 #include "common.h"
 #include "kernels.h"
 
@@ -31,17 +34,17 @@ namespace mlstm {
 namespace {
 
 struct HvItem {
-  int bh, c, ch;               // (batch * head), chunk, group of 256 value columns
+  int bh, c, ch;               // (batch * head), chunk, group of 512 value columns
   int slot;                    // kept boundary state the chunk uses
   int sc_first, sc_step, nsc;  // source chunks: sc_first, sc_first + sc_step, ... (nsc of them, the own chunk last)
 };
 
-// Work item of workgroup `vid` in round `round`.  Consecutive workgroups take consecutive items (the column groups of
-// a chunk, then the next chunk: they share rows and kept states through the L2 of their XCD); the assignment rotates
-// by one chunk per round so that a workgroup does not always get the chunks with the same number of source chunks.
+// Work item of workgroup `vid` in round `round`.  Consecutive workgroups take consecutive items (neighbouring chunks
+// share rows and kept states through the L2 of their XCD); the assignment rotates by one item per round so that a
+// workgroup does not always get the chunks with the same number of source chunks.
 template <bool IS_DV>
 __device__ __forceinline__ bool hv_decode(HvItem& it, int round, int vid, int G, int n_items, int NC, int NCH, int stride) {
-  const int rot = (vid + round * NCH) % G;
+  const int rot = (vid + round) % G;
   const long long idx = (long long)round * G + rot;
   if (idx >= n_items) return false;
   const int i = (int)idx;
@@ -63,6 +66,8 @@ __device__ __forceinline__ bool hv_decode(HvItem& it, int round, int vid, int G,
   return true;
 }
 
+constexpr float kLog2e = 1.4426950408889634f;
+
 }  // namespace
 
 #ifdef HV_EXP_TIMING
@@ -75,34 +80,39 @@ __device__ unsigned long long g_hv_dbg[32];
     dbg_wait += t1_ - t0_;                                            \
     dbg_n += 1;                                                       \
   }
-#define HV_PHASE(k)
 #define HV_TB(k) unsigned long long treg_##k = 0; if ((k) == HV_T_REGION) treg_##k = __builtin_amdgcn_s_memrealtime();
 #define HV_TE(k) if ((k) == HV_T_REGION) { dbg_reg += __builtin_amdgcn_s_memrealtime() - treg_##k; dbg_regn += 1; }
 #else
 #define HV_SYNC() __syncthreads()
-#define HV_PHASE(k)
 #define HV_TB(k)
 #define HV_TE(k)
 #endif
+
 template <bool IS_DV, bool F16>
-__global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_items, int n_rounds) {
+__global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items, int n_rounds) {
   constexpr int DHQK = 256;
   constexpr int QS = DHQK + 8;   // resident rows [128][DHQK] and score-operand slabs [64][DHQK], fragment order
-  constexpr int VS = 256 + 16;   // value-operand slab: 64 rows x 256 value columns, row-major
+  constexpr int VS = 512 + 16;   // value-operand slab: 32 rows x 512 value columns, row-major
   constexpr int PSS = 64 + 8;    // gated score block P[n][o]: 128 positions x 64 source positions
-  constexpr int SLOT = 64 * VS;  // elements per ring slot (the largest slab kind)
+  constexpr int SLOT = 64 * QS;  // elements per ring slot (the largest slab kind)
   constexpr int ND = DHQK / 16;
-  static_assert(64 * QS <= SLOT && 16384 <= SLOT, "every slab kind fits a ring slot");
+  static_assert(32 * VS <= SLOT && 16384 <= SLOT, "every slab kind fits a ring slot");
   extern __shared__ __align__(16) unsigned char smem_raw[];
+  // [resident rows | ring slot 0 | score block | ring slot 1 | vectors]: the epilogue stages through everything between
+  // the resident rows and the vectors in its first step and through score block + slot 1 in its second (slot 0 then
+  // receives the first state slab)
   uint16_t* const Ns = (uint16_t*)smem_raw;
-  uint16_t* const Ps = Ns + 128 * QS;
-  uint16_t* const Ring = Ps + 128 * PSS;
-  float* const rows = (float*)(Ring + 2 * SLOT);  // [4][128] partial row sums of the own chunk's scores (forward)
-  float* const inv = rows + 4 * 128;              // [128] forward: 1 / (row normaliser + eps)
-  float* const nperm = inv + 128;                 // [DHQK] forward: n before the chunk, fragment order
-  float* const ovec = nperm + DHQK;               // [64] gate vector of the source half: w_j (forward) / u_t (dV)
-  float* const orho = ovec + 64;                  // [64] dV: rho_t of the source half
-  constexpr uint32_t kRingOff = (128 * QS + 128 * PSS) * 2;
+  uint16_t* const Ring0 = Ns + 128 * QS;
+  uint16_t* const Ps = Ring0 + SLOT;
+  uint16_t* const Ring1 = Ps + 128 * PSS;
+  float* const rows = (float*)(Ring1 + SLOT);  // [4][128] partial row sums of the own chunk's scores (forward)
+  float* const inv = rows + 4 * 128;           // [128] forward: 1 / (row normaliser + eps)
+  float* const nperm = inv + 128;              // [DHQK] forward: n before the chunk, fragment order
+  float* const ovec = nperm + DHQK;            // [64] gate vector of the source half times log2(e): w_j (forward) / u_t (dV)
+  float* const orho = ovec + 64;               // [64] dV: rho_t of the source half
+  float* const denq = orho + 64;               // [128] forward: bbar_t / sqrt(d) * (q_t . n_prev), the inter-chunk part of the denominator
+  float* const mcv = denq + 128;               // [128] forward: combined stabiliser of the item's positions
+  constexpr uint32_t kRing0Off = 128 * QS * 2, kRing1Off = kRing0Off + (SLOT + 128 * PSS) * 2;
 
 #ifdef HV_EXP_TIMING
   unsigned long long dbg_wait = 0, dbg_n = 0;
@@ -114,7 +124,7 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
   const int G = gridDim.x;
   int vid = blockIdx.x;
   if (G % 8 == 0) vid = (vid % 8) * (G / 8) + vid / 8;  // consecutive ids share an XCD (and its L2)
-  const int NC = a.NC, S = a.S, DHHV = a.DHHV, NCH = DHHV / 256, stride = a.stride;
+  const int NC = a.NC, S = a.S, DHHV = a.DHHV, NCH = DHHV / 512, stride = a.stride;
   const size_t Sp = (size_t)NC * kChunk;
   const int NCS = (NC + stride - 1) / stride;
 
@@ -124,15 +134,15 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
     // L - 3 (the consumers are done with slab L - 4, whose ring slot slab L - 2 goes into), write slab L - 2 from the
     // register set to LDS, request slab L into the set.  The destination in LDS travels with the data: byte offset of
     // the thread's first piece | slab kind << 20 (0 fragment-order rows, 1 state fragments, 3 value rows) | gate-vector
-    // flag << 22; the thread's other three pieces lie a fixed distance apart.
-    const int p = (wave_all - 8) * 64 + lane;  // 0 .. 511: every thread moves four 16-byte pieces of every slab
+    // flag << 22; the thread's other seven pieces lie a fixed distance apart.
+    const int p = (wave_all - 8) * 64 + lane;  // 0 .. 255: every thread moves eight 16-byte pieces of every slab
     const char* const Xn_b = (const char*)(IS_DV ? a.K : a.Q);
     const char* const Xo_b = (const char*)(IS_DV ? a.Q : a.K);
     const char* const Xw_b = (const char*)(IS_DV ? a.dH : a.V);
     const char* const St_b = (const char*)a.states;
     const float* const ov_src = IS_DV ? a.g.u : a.g.w;
     const float* const rho_src = (IS_DV && a.use_nrow) ? a.nrow : ov_src;
-    uint4 fd[2][4];
+    uint4 fd[2][8];
     uint32_t fw[2];
     float fa[2][2];
     int L = 0;
@@ -142,32 +152,24 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
     const uint32_t kind_ = (uint32_t)__builtin_amdgcn_readfirstlane((int)((w_ >> 20) & 3));                          \
     const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
     const uint32_t half_ = kind_ == 0 ? 16u : 8u;                                                                    \
-    const uint32_t step_ = kind_ == 0 ? 16 * QS * 2 : (kind_ == 1 ? 8192 : 16 * VS * 2);                             \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                               \
+    const uint32_t step_ = kind_ == 0 ? 8 * QS * 2 : (kind_ == 1 ? 4096 : 4 * VS * 2);                               \
+    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) {                                                               \
       *(uint2*)(smem_raw + d0_ + i_ * step_) = make_uint2(fd[E][i_].x, fd[E][i_].y);                                 \
       *(uint2*)(smem_raw + d0_ + i_ * step_ + half_) = make_uint2(fd[E][i_].z, fd[E][i_].w);                         \
     }                                                                                                                \
     if (__builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 64) {                                           \
-      ovec[p] = fa[E][0];                                                                                            \
+      ovec[p] = fa[E][0] * kLog2e;                                                                                   \
       if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa[E][1] + a.eps) : 1.f;                                              \
     }                                                                                                                \
   }
     // base_: (batch, head) base of the operand; g0_: byte offset of the thread's first piece, gs_: distance between
     // its pieces; gi_: index of the gate-vector entry that rides along (stored only with the flag set; the other
     // slabs request an entry all the same so that every step issues the same loads)
-#define HV_PROC(E, base_, g0_, gs_, dstw_, gi_)                                                                      \
-  {                                                                                                                  \
-    if (L >= 3) HV_SYNC();                                                                                     \
-    HV_TB(6) if (L >= 2) HV_STORE(E) HV_TE(6)                                                                         \
-    HV_TB(7) HV_EXP_LOADS(E, base_, g0_, gs_, gi_) HV_TE(7)                                                           \
-    fw[E] = (dstw_);                                                                                                 \
-    ++L;                                                                                                             \
-  }
 #ifdef HV_EXP_NOLOAD
 #define HV_EXP_LOADS(E, base_, g0_, gs_, gi_)                                                                        \
   {                                                                                                                  \
     fa[E][0] = (float)(g0_); fa[E][1] = 1.f;                                                                         \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd[E][i_] = make_uint4((g0_) + i_ * (gs_), 0, 0, 0);            \
+    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) fd[E][i_] = make_uint4((g0_) + i_ * (gs_), 0, 0, 0);            \
     (void)(base_); (void)(gi_);                                                                                      \
   }
 #else
@@ -175,14 +177,22 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
   {                                                                                                                  \
     fa[E][0] = ov_src[gi_];                                                                                          \
     fa[E][1] = rho_src[gi_];                                                                                         \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd[E][i_] = *(const uint4*)((base_) + ((g0_) + i_ * (gs_)));    \
+    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) fd[E][i_] = *(const uint4*)((base_) + ((g0_) + i_ * (gs_)));    \
   }
 #endif
+#define HV_PROC(E, base_, g0_, gs_, dstw_, gi_)                                                                      \
+  {                                                                                                                  \
+    if (L >= 3) HV_SYNC();                                                                                           \
+    HV_TB(6) if (L >= 2) HV_STORE(E) HV_TE(6)                                                                        \
+    HV_TB(7) HV_EXP_LOADS(E, base_, g0_, gs_, gi_) HV_TE(7)                                                          \
+    fw[E] = (dstw_);                                                                                                 \
+    ++L;                                                                                                             \
+  }
     HvItem it;
     for (int rd = 0; rd < n_rounds; ++rd) {
       if (!hv_decode<IS_DV>(it, rd, vid, G, n_items, NC, NCH, stride)) continue;
       const uint32_t pl = (uint32_t)opaque(p);
-      const uint32_t row = pl >> 5, pc = pl & 31;  // rows of 512 bytes: 32 pieces per row, 16 rows per sweep
+      const uint32_t row = pl >> 5, pc = pl & 31;  // rows of 512 bytes: 32 pieces per row, 8 rows per sweep
       const size_t gown = (size_t)it.bh * Sp + (size_t)it.c * kChunk + (pl & 63);
       // fragment-order destination of piece pc inside a row (see store_perm16)
       const uint32_t permo = (pc >> 1) * 32 + 8 * (pc & 1);
@@ -191,32 +201,39 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
         const char* const base = Xn_b + (size_t)it.bh * S * DHQK * 2;
         const uint32_t g0 = ((uint32_t)(it.c * kChunk) + row) * (DHQK * 2) + pc * 16;
         const uint32_t d0 = row * (QS * 2) + permo;
-        HV_PROC(0, base, g0, 16 * DHQK * 2, d0, gown)
-        HV_PROC(1, base, g0 + 64 * DHQK * 2, 16 * DHQK * 2, d0 + 64 * QS * 2, gown)
+        HV_PROC(0, base, g0, 8 * DHQK * 2, d0, gown)
+        HV_PROC(1, base, g0 + 64 * DHQK * 2, 8 * DHQK * 2, d0 + 64 * QS * 2, gown)
       }
       {
-        // ---- state fragments: slab si holds contraction steps 4 si .. 4 si + 3 of the eight 32-column blocks
+        // ---- state fragments: slab si holds contraction steps 2 si, 2 si + 1 of the sixteen 32-column blocks
         const char* const base = St_b + ((size_t)it.bh * NCS + it.slot) * (size_t)(DHHV / 32) * ND * 1024;
-        const uint32_t wbl = pl >> 8, dsl = (pl >> 6) & 3;
-        const uint32_t g0 = (((uint32_t)it.ch * 8 + wbl) * ND + dsl) * 1024 + (pl & 63) * 16;
-        for (int si = 0; si < 4; si += 2) {
-          HV_PROC(0, base, g0 + si * 4096, 2 * ND * 1024, (kRingOff + pl * 16) | (1u << 20), gown)
-          HV_PROC(1, base, g0 + (si + 1) * 4096, 2 * ND * 1024, (kRingOff + SLOT * 2 + pl * 16) | (1u << 20), gown)
+        const uint32_t f0 = pl >> 6;  // fragment of the first piece inside the slab: block f0 / 2, contraction step f0 % 2
+        const uint32_t g0 = (((uint32_t)it.ch * 16 + (f0 >> 1)) * ND + (f0 & 1)) * 1024 + (pl & 63) * 16;
+        for (int si = 0; si < 8; si += 2) {
+          HV_PROC(0, base, g0 + si * 2048, 2 * ND * 1024, (kRing0Off + pl * 16) | (1u << 20), gown)
+          HV_PROC(1, base, g0 + (si + 1) * 2048, 2 * ND * 1024, (kRing1Off + pl * 16) | (1u << 20), gown)
         }
       }
       {
         const char* const kbase = Xo_b + (size_t)it.bh * S * DHQK * 2;
         const char* const vbase = Xw_b + (size_t)it.bh * S * DHHV * 2;
-        const uint32_t kd0 = kRingOff + row * (QS * 2) + permo;
-        const uint32_t vd0 = (kRingOff + SLOT * 2 + row * (VS * 2) + pc * 16) | (3u << 20);
+        const uint32_t kd = row * (QS * 2) + permo;
+        const uint32_t vrow = pl >> 6, vpc = pl & 63;  // rows of 1024 bytes: 64 pieces per row, 4 rows per sweep
+        const uint32_t vd = (vrow * (VS * 2) + vpc * 16) | (3u << 20);
         for (int sci = 0; sci < it.nsc; ++sci) {
           const int sc = it.sc_first + sci * it.sc_step;
-          for (int kh = 0; kh < 2; ++kh) {
-            const uint32_t t0 = (uint32_t)(sc * kChunk + 64 * kh) + row;
-            const size_t gi = (size_t)it.bh * Sp + (size_t)sc * kChunk + 64 * kh + (pl & 63);
-            HV_PROC(0, kbase, t0 * (DHQK * 2) + pc * 16, 16 * DHQK * 2, kd0 | (1u << 22), gi)
-            HV_PROC(1, vbase, t0 * (uint32_t)(DHHV * 2) + (uint32_t)it.ch * 512 + pc * 16, 16 * (uint32_t)DHHV * 2, vd0, gown)
-          }
+          const uint32_t t0 = (uint32_t)(sc * kChunk);
+          const size_t gi = (size_t)it.bh * Sp + (size_t)sc * kChunk + (pl & 63);
+          const uint32_t vg = (t0 + vrow) * (uint32_t)(DHHV * 2) + (uint32_t)it.ch * 1024 + vpc * 16;
+          const uint32_t vgs = 4 * (uint32_t)DHHV * 2, vg32 = 32 * (uint32_t)DHHV * 2;
+          // first half: scores -> set 0 / slot 0, value rows -> set 1 / slot 1 and set 0 / slot 0
+          HV_PROC(0, kbase, (t0 + row) * (DHQK * 2) + pc * 16, 8 * DHQK * 2, (kRing0Off + kd) | (1u << 22), gi)
+          HV_PROC(1, vbase, vg, vgs, kRing1Off + vd, gown)
+          HV_PROC(0, vbase, vg + vg32, vgs, kRing0Off + vd, gown)
+          // second half: the other way round
+          HV_PROC(1, kbase, (t0 + 64 + row) * (DHQK * 2) + pc * 16, 8 * DHQK * 2, (kRing1Off + kd) | (1u << 22), gi + 64)
+          HV_PROC(0, vbase, vg + 2 * vg32, vgs, kRing0Off + vd, gown)
+          HV_PROC(1, vbase, vg + 3 * vg32, vgs, kRing1Off + vd, gown)
         }
       }
     }
@@ -240,16 +257,13 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
 #else
 #define HV_MFMA(C_, A_, B_) mfma32<F16>(C_, A_, B_)
 #endif
-#ifdef HV_EXP_PRIO
-    __builtin_amdgcn_s_setprio(HV_EXP_PRIO);
-#endif
     const int wave = wave_all;
     const int tid = wave * 64 + lane;
-    const int pi = wave & 1, ci = wave >> 1;  // output role: positions 64 pi .., value columns 64 ci .. of the item
+    const int pi = wave & 1, ci = wave >> 1;  // output role: positions 64 pi .., value columns 128 ci .. of the item
     const int pb = wave & 3, kb = wave >> 2;  // score role: position block pb, source block kb of a 64-position half
-    f32x16 acc[2][2], sacc;
+    f32x16 acc[4][2], sacc;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -257,29 +271,30 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
     HvItem it, prev;
     prev = HvItem{0, 0, 0, 0, 0, 1, 1};
     bool have_prev = false;
-    // The accumulators are only ever touched in straight-line code between barriers: no matrix instruction sits under
-    // a condition (dead score blocks of the own chunk are multiplied and masked to zero by the gating), so the
-    // compiler keeps every accumulator in one place.  The epilogue is a macro with a literal position block:
-    // (normalise,) round, transpose 32 positions x 64 columns through a private part of the idle score block,
-    // coalesced non-temporal stores.
-#define HV_EPILOGUE(NB)                                                                                              \
+    // The accumulators are only ever touched in straight-line code between barriers: no matrix instruction that
+    // updates them sits under a condition (dead score blocks of the own chunk are masked to zero by the gating), so
+    // the compiler keeps every accumulator in one place.  The epilogue is a macro with literal block indices:
+    // (normalise,) round, transpose 32 positions x (32 NMB) columns through a private staging area, coalesced
+    // non-temporal stores.  STG_: staging base of this wave, MB0_: first column block, NMB_: column blocks (4 or 2).
+#define HV_EPILOGUE(NB, MB0_, NMB_, STG_)                                                                            \
   {                                                                                                                  \
     const int le = opaque(lane);                                                                                     \
     const int r = le & 31, h = le >> 5;                                                                              \
-    constexpr int SR = 64 + 8; /* staging row: 64 value columns */                                                   \
-    uint16_t* const stg = Ps + (wave & 3) * (32 * SR);                                                               \
+    constexpr int SR = 32 * (NMB_) + 8; /* staging row */                                                            \
+    uint16_t* const stg = (STG_);                                                                                    \
     const float iv = IS_DV ? 1.f : inv[64 * pi + 32 * NB + r];                                                       \
-    _Pragma("unroll") for (int mb = 0; mb < 2; ++mb) _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {              \
+    _Pragma("unroll") for (int mb = 0; mb < (NMB_); ++mb) _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {         \
       *(uint2*)(stg + r * SR + 32 * mb + 8 * g4 + 4 * h) =                                                           \
-          make_uint2(pack2<F16>(acc[mb][NB][4 * g4 + 0] * iv, acc[mb][NB][4 * g4 + 1] * iv),                         \
-                     pack2<F16>(acc[mb][NB][4 * g4 + 2] * iv, acc[mb][NB][4 * g4 + 3] * iv));                        \
+          make_uint2(pack2<F16>(acc[(MB0_) + mb][NB][4 * g4 + 0] * iv, acc[(MB0_) + mb][NB][4 * g4 + 1] * iv),       \
+                     pack2<F16>(acc[(MB0_) + mb][NB][4 * g4 + 2] * iv, acc[(MB0_) + mb][NB][4 * g4 + 3] * iv));      \
     }                                                                                                                \
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                           \
     __builtin_amdgcn_wave_barrier();                                                                                 \
     uint16_t* const Og = a.Out + ((size_t)prev.bh * S + (size_t)prev.c * kChunk + 64 * pi + 32 * NB) * DHHV +        \
-                         prev.ch * 256 + 64 * ci;                                                                    \
-    _Pragma("unroll") for (int k = 0; k < 4; ++k) {                                                                  \
-      const int row = (le >> 3) + 8 * k, pc = le & 7;                                                                \
+                         prev.ch * 512 + 128 * ci + 32 * (MB0_);                                                     \
+    constexpr int VPR = 4 * (NMB_); /* 16-byte vectors per row */                                                    \
+    _Pragma("unroll") for (int k = 0; k < 32 * VPR / 64; ++k) {                                                      \
+      const int row = le / VPR + (64 / VPR) * k, pc = le % VPR;                                                      \
       __builtin_nontemporal_store(*(const u32x4*)(stg + row * SR + pc * 8), (u32x4*)(Og + (size_t)row * DHHV + pc * 8)); \
     }                                                                                                                \
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                           \
@@ -291,15 +306,13 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
       const size_t hofs = (size_t)bh * Sp, gofs = hofs + (size_t)c * kChunk;
       const float* graw = a.g.graw + (size_t)bh * NC;
       const float* mst = a.g.mstates + (size_t)bh * (NC + 1);
-      // ---- two steps while the resident rows arrive: the previous item's output leaves (waves 0..3 in the first
-      // step, 4..7 in the second: the staging area holds four tiles), the per-item vectors are requested
-      float csr[2], nv, cs0r = 0.f, mcr = 0.f, np0 = 0.f, np1 = 0.f, np2 = 0.f, qn = 0.f;
+      // ---- two steps while the resident rows arrive: the previous item's output leaves (the first 32 of a wave's 64
+      // positions, then the other 32 in two rounds of 64 columns: the second step has less LDS to stage through), the
+      // per-item vectors are requested
+      float csr[2], nv, cs0r = 0.f, mcr = 0.f, np0 = 0.f, np1 = 0.f, np2 = 0.f;
       HV_SYNC();
       HV_TB(5)
-      if (have_prev && wave < 4) {
-        HV_EPILOGUE(0)
-        HV_EPILOGUE(1)
-      }
+      if (have_prev) HV_EPILOGUE(0, 0, 4, Ring0 + wave * (32 * 136))
       {
         const int r = opaque(lane) & 31;
         float gsum = 0.f, xs = 1.f;
@@ -333,32 +346,17 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
       }
       HV_TE(5)
       HV_SYNC();
-      if (have_prev && wave >= 4) {
-        HV_EPILOGUE(0)
-        HV_EPILOGUE(1)
+      if (have_prev) {
+        HV_EPILOGUE(1, 0, 2, Ps + wave * (32 * 72))
+        HV_EPILOGUE(1, 2, 2, Ps + wave * (32 * 72))
       }
-      // ---- inter-chunk product: Out^T = State^T Xn^T, four contraction steps per slab
+      if (!IS_DV && tid < DHQK) nperm[perm16(tid)] = (np0 + np1) + np2;
+      // ---- inter-chunk product: Out^T = State^T Xn^T, two contraction steps per slab
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
-      // (the operand fragments that do not depend on the incoming slab -- resident rows -- are requested before the
-      // barrier of a step, while the wave would otherwise only wait)
-      Frag Bpre[2];
-      {
-        const int le = opaque(lane);
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb) Bpre[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + (le & 31)) * QS + 8 * (le >> 5));
-      }
-#pragma unroll
-      for (int si = 0; si < 4; ++si) {
+      for (int si = 0; si < 8; ++si) {
         HV_SYNC();
-        HV_PHASE(1)
         if (!IS_DV) {
-          if (si == 0 && tid < DHQK) nperm[perm16(tid)] = (np0 + np1) + np2;
-          if (si == 1) {
+          if (si == 0) {
             // forward: q_t . n_prev for the denominators (four threads per position), while the resident rows are
             // all there -- the next item's rows start to arrive during this item's last step
             const int td = opaque(tid);
@@ -366,7 +364,7 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
             const uint16_t* qrow = Ns + t * QS + part * (DHQK / 4);
             const float* np = nperm + part * (DHQK / 4);
             float dot = 0.f;
-#pragma unroll 2
+#pragma unroll 1
             for (int d = 0; d < DHQK / 4; d += 8) {
               const uint4 qv = *(const uint4*)(qrow + d);
               const float4 na = *(const float4*)(np + d), nb4 = *(const float4*)(np + d + 4);
@@ -375,38 +373,49 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
             }
             dot += __shfl_xor(dot, 1);
             dot += __shfl_xor(dot, 2);
-            qn = dot;
+            // parked in LDS until the row sums of the own chunk are complete: registers are what this kernel is short of
+            if (part == 0) {
+              denq[t] = cs0r * dot;
+              mcv[t] = mcr;
+            }
           }
+        }
+        if (si == 0) {
+          // (after the dot product above, which runs while no accumulator is live)
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
         }
         HV_TB(1)
         const int le = opaque(lane);
         const int r = le & 31, h = le >> 5;
-        const uint16_t* const slab = Ring + (si & 1) * SLOT;
+        const uint16_t* const slab = (si & 1) ? Ring1 : Ring0;
 #pragma unroll
-        for (int dsl = 0; dsl < 4; ++dsl) {
-          Frag A[2], B[2];
+        for (int dsl = 0; dsl < 2; ++dsl) {
+          Frag A[4], B[2];
 #pragma unroll
-          for (int mb = 0; mb < 2; ++mb) A[mb].u = *(const uint4*)(slab + ((2 * ci + mb) * 4 + dsl) * 512 + le * 8);
+          for (int mb = 0; mb < 4; ++mb) A[mb].u = *(const uint4*)(slab + ((4 * ci + mb) * 2 + dsl) * 512 + le * 8);
 #pragma unroll
-          for (int nb = 0; nb < 2; ++nb) {
-            if (dsl == 0) B[nb] = Bpre[nb];
-            else B[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + r) * QS + 16 * (4 * si + dsl) + 8 * h);
-          }
+          for (int nb = 0; nb < 2; ++nb)
+            B[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + r) * QS + 16 * (2 * si + dsl) + 8 * h);
 #pragma unroll
-          for (int mb = 0; mb < 2; ++mb)
+          for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) HV_MFMA(acc[mb][nb], A[mb], B[nb]);
         }
-        if (si < 3) {
-#pragma unroll
-          for (int nb = 0; nb < 2; ++nb) Bpre[nb].u = *(const uint4*)(Ns + (64 * pi + 32 * nb + r) * QS + 16 * (4 * si + 4) + 8 * h);
-        }
         HV_TE(1)
       }
+      // (kept apart from the matrix instructions around it: interleaved with them the products land in fresh
+      // registers, a second copy of an accumulator tile the register file has no room for)
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= csr[nb];
+        for (int mb = 0; mb < 4; ++mb) acc[mb][nb] *= csr[nb];
+      __builtin_amdgcn_sched_barrier(0);
 
       // ---- source chunks (the own chunk last), 64 source positions at a time
       for (int sci = 0; sci < it.nsc; ++sci) {
@@ -414,36 +423,35 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
         const bool own = sc == c;
         float gs = 0.f;  // decay between the source chunk and this chunk
         for (int x = (IS_DV ? c : sc); x < (IS_DV ? sc : c); ++x) gs += graw[x];
+        // exponent offset of this lane's position, in powers of two, with the 1/sqrt(d) of the scores folded in
+        const float un2 = (nv + (IS_DV ? -gs : gs)) * kLog2e + (IS_DV ? -1.f : 1.f) * __log2f(a.qk_scale);
+#pragma unroll
         for (int kh = 0; kh < 2; ++kh) {
+          // the two halves use the ring slots the other way round (three slabs per half)
+          const uint16_t* const kslab = kh == 0 ? Ring0 : Ring1;
           // scores of position block pb against source block kb of this half
 #pragma unroll
           for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-          Frag Bk[4];
-          {
-            const int le = opaque(lane);
-#pragma unroll
-            for (int ds = 0; ds < 4; ++ds) Bk[ds].u = *(const uint4*)(Ns + (32 * pb + (le & 31)) * QS + 16 * ds + 8 * (le >> 5));
-          }
           HV_SYNC();
-          HV_PHASE(2)
           {
             HV_TB(2)
             const int le = opaque(lane);
             const int r = le & 31, h = le >> 5;
-            const uint16_t* const slab = Ring;
+            // blocks of the own chunk that the causal mask empties are not multiplied (their rows stay zero)
+            const bool live = !own || (IS_DV ? (2 * kh + kb >= pb) : (2 * kh + kb <= pb));
+            if (live) {
 #pragma unroll
-            for (int ds = 0; ds < ND; ++ds) {
-              Frag A, B;
-              A.u = *(const uint4*)(slab + (32 * kb + r) * QS + 16 * ds + 8 * h);
-              if (ds < 4) B = Bk[ds];
-              else B.u = *(const uint4*)(Ns + (32 * pb + r) * QS + 16 * ds + 8 * h);
-              HV_MFMA(sacc, A, B);
+              for (int ds = 0; ds < ND; ++ds) {
+                Frag A, B;
+                A.u = *(const uint4*)(kslab + (32 * kb + r) * QS + 16 * ds + 8 * h);
+                B.u = *(const uint4*)(Ns + (32 * pb + r) * QS + 16 * ds + 8 * h);
+                HV_MFMA(sacc, A, B);
+              }
             }
             HV_TE(2)
             HV_TB(3)
             // gate, mask, round and write P as Ps[n][o]; forward: fp32 row sums over the own chunk's positions
             const int n = 32 * pb + r;  // position inside the chunk
-            const float un = nv + (IS_DV ? -gs : gs);
             float rsum = 0.f;
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
@@ -459,9 +467,11 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
 #pragma unroll
               for (int q = 0; q < 4; ++q) {
                 const int o = 64 * kh + ol + q;
-                const float ex = IS_DV ? (xov[q] - un) : (un - xov[q]);
+                // exp(u_t - w_j + G) / sqrt(d) as one power of two
+                const float e2 = __builtin_amdgcn_exp2f(IS_DV ? (xov[q] - un2) : (un2 - xov[q]));
                 const bool keep = !own || (IS_DV ? (n <= o) : (o <= n));
-                const float val = sacc[4 * g4 + q] * a.qk_scale * __expf(ex) * rho[q];
+                float val = sacc[4 * g4 + q] * e2;
+                if (IS_DV) val *= rho[q];
                 pv[q] = keep ? val : 0.f;
                 rsum += pv[q];
               }
@@ -473,42 +483,43 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
             }
             HV_TE(3)
           }
-          // Out^T += Xw^T P over the 64 source positions of the half
-          HV_SYNC();
-          HV_PHASE(3)
-          {
+          // Out^T += Xw^T P over the 64 source positions of the half: two slabs of 32
+#pragma unroll
+          for (int vi = 0; vi < 2; ++vi) {
+            HV_SYNC();
+            HV_TB(4)
             const int le = opaque(lane);
             const int r = le & 31, h = le >> 5;
             const int q16 = (le >> 4) & 1, i16 = le & 15;
             const int krow = 8 * h + (i16 >> 2), ncol = 16 * q16 + 4 * (i16 & 3);
-            HV_TB(4)
-            const uint16_t* const slab = Ring + SLOT;
+            const uint16_t* const slab = ((kh + vi) & 1) ? Ring0 : Ring1;
 #pragma unroll
-            for (int k16 = 0; k16 < 4; ++k16) {
-              Frag A[2], B[2];
+            for (int k16 = 0; k16 < 2; ++k16) {
+              Frag A[4], B[2];
 #pragma unroll
-              for (int mb = 0; mb < 2; ++mb) {
-                const uint16_t* pp = slab + (16 * k16 + krow) * VS + (64 * ci + 32 * mb + ncol);
+              for (int mb = 0; mb < 4; ++mb) {
+                const uint16_t* pp = slab + (16 * k16 + krow) * VS + (128 * ci + 32 * mb + ncol);
                 A[mb].d[0] = lds_read_tr16(pp);
                 A[mb].d[1] = lds_read_tr16(pp + 4 * VS);
               }
 #pragma unroll
               for (int nb = 0; nb < 2; ++nb)
-                B[nb].u = *(const uint4*)(Ps + (64 * pi + 32 * nb + r) * PSS + 16 * k16 + 8 * h);
+                B[nb].u = *(const uint4*)(Ps + (64 * pi + 32 * nb + r) * PSS + 32 * vi + 16 * k16 + 8 * h);
 #pragma unroll
-              for (int mb = 0; mb < 2; ++mb)
+              for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) HV_MFMA(acc[mb][nb], A[mb], B[nb]);
             }
             HV_TE(4)
             // ---- forward: denominators, once all row sums of the own chunk are there (it is the last source chunk)
-            if (!IS_DV && own && kh == 1) {
+            if (!IS_DV && own && kh == 1 && vi == 1) {
               const int td = opaque(tid);
               const int t = td >> 2;
               if ((td & 3) == 0) {
                 float nmax = 1.f, iv = 1.f;
+                const float mcr = mcv[t];
                 if (a.use_nrow) {
-                  float den = cs0r * qn;
+                  float den = denq[t];
 #pragma unroll
                   for (int b4 = 0; b4 < 4; ++b4) den += rows[b4 * 128 + t];
                   const float floor_v = a.sig_gate ? 1.f : __expf(-mcr);
@@ -532,15 +543,10 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
     }
     if (have_prev) {
       HV_SYNC();
-      if (wave < 4) {
-        HV_EPILOGUE(0)
-        HV_EPILOGUE(1)
-      }
+      HV_EPILOGUE(0, 0, 4, Ring0 + wave * (32 * 136))
       HV_SYNC();
-      if (wave >= 4) {
-        HV_EPILOGUE(0)
-        HV_EPILOGUE(1)
-      }
+      HV_EPILOGUE(1, 0, 2, Ps + wave * (32 * 72))
+      HV_EPILOGUE(1, 2, 2, Ps + wave * (32 * 72))
     }
 #undef HV_EPILOGUE
 #undef HV_MFMA
@@ -558,7 +564,7 @@ __global__ __launch_bounds__(1024) void stream_hv_kernel(ParHvArgs a, int n_item
 }
 
 bool stream_hv_supported(const ParHvArgs& a) {
-  return a.DHQK == 256 && a.DHHV % 256 == 0 && a.S % kChunk == 0 && a.head_norm == 0;
+  return a.DHQK == 256 && a.DHHV % 512 == 0 && a.S % kChunk == 0 && a.head_norm == 0;
 }
 
 namespace {
@@ -576,9 +582,9 @@ int device_cu_count() {
 
 template <bool IS_DV, bool F16>
 const char* launch_stream_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
-  constexpr int QS = 256 + 8, PSS = 72, SLOT = 64 * 272;
-  const size_t smem = (size_t)(128 * QS + 128 * PSS + 2 * SLOT) * 2 + (size_t)(4 * 128 + 128 + 256 + 64 + 64) * 4;
-  const long long n_items = (long long)BH * a.NC * (a.DHHV / 256);
+  constexpr int QS = 256 + 8, PSS = 72, SLOT = 64 * QS;
+  const size_t smem = (size_t)(128 * QS + 128 * PSS + 2 * SLOT) * 2 + (size_t)(4 * 128 + 128 + 256 + 64 + 64 + 128 + 128) * 4;
+  const long long n_items = (long long)BH * a.NC * (a.DHHV / 512);
   if (n_items >= (1ll << 31)) return "stream_hv: too many work items";
   if ((size_t)a.S * (size_t)a.DHHV * 2 >= ((size_t)1 << 32)) return "stream_hv: one (batch, head) slab of an input exceeds 4 GiB";
   const int cus = device_cu_count();
@@ -589,13 +595,13 @@ const char* launch_stream_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
   if (hipFuncSetAttribute((const void*)stream_hv_kernel<IS_DV, F16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
       hipSuccess)
     return "stream_hv: cannot raise the dynamic LDS limit";
-  hipLaunchKernelGGL((stream_hv_kernel<IS_DV, F16>), dim3(G), dim3(1024), smem, stream, a, (int)n_items, n_rounds);
+  hipLaunchKernelGGL((stream_hv_kernel<IS_DV, F16>), dim3(G), dim3(768), smem, stream, a, (int)n_items, n_rounds);
   return nullptr;
 }
 }  // namespace
 
 const char* launch_stream_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
-  if (!stream_hv_supported(a)) return "stream_hv: unsupported shape (needs DHQK = 256, DHHV % 256 == 0, S % 128 == 0, no head norm)";
+  if (!stream_hv_supported(a)) return "stream_hv: unsupported shape (needs DHQK = 256, DHHV % 512 == 0, S % 128 == 0, no head norm)";
   if (a.stride < 1 || a.stride > kMaxStateStride) return "stream_hv: state stride out of range";
   if (is_dv) return a.f16 ? launch_stream_hv_t<true, true>(a, BH, stream) : launch_stream_hv_t<true, false>(a, BH, stream);
   return a.f16 ? launch_stream_hv_t<false, true>(a, BH, stream) : launch_stream_hv_t<false, false>(a, BH, stream);
