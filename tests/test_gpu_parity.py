@@ -31,12 +31,14 @@ DEV = "cuda"
 _VARIANT = {"kernel_path": "auto", "chunk_size_intra": None}
 
 
-@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "fused-1"])
+@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "stream-1", "stream-2", "stream-4", "fused-1"])
 def kernel_variant(request):
     """Every test runs once per kernel variant of the chunkwise passes: the split path (state scan + chunk-parallel
-    kernels) with a chunk state kept every 1, 2 or 4 chunks, and the fused path (sequential kernels with a
-    register-resident state; head dimensions it does not support are skipped; stride 1, so that all its kernels group
-    the products the same way -- the fused path with other strides is part of the randomised sweep)."""
+    kernels) with a chunk state kept every 1, 2 or 4 chunks, the stream path (the same scans, chunk-parallel kernels
+    as persistent workgroups with producer and consumer waves; shapes it does not support are skipped), and the fused
+    path (sequential kernels with a register-resident state; head dimensions it does not support are skipped; stride
+    1, so that all its kernels group the products the same way -- the fused path with other strides is part of the
+    randomised sweep)."""
     path, stride = request.param.split("-")
     _VARIANT.update(kernel_path=path, chunk_size_intra=128 * int(stride))
     yield request.param
@@ -56,6 +58,8 @@ def _with_variant(op):
         except RuntimeError as e:
             if "fused kernel path supports" in str(e):
                 pytest.skip("the fused path does not support these head dimensions")
+            if "stream kernel path supports" in str(e):
+                pytest.skip("the stream path does not support this shape")
             raise
 
     call.supports_any_sequence_length = True
@@ -68,6 +72,14 @@ def _ops():
 
     return (_with_variant(mlstm_chunkwise__hip_xl_chunk), _with_variant(mlstm_siging_chunkwise__hip_xl_chunk),
             mlstm_recurrent_step__hip, mlstm_recurrent_sequence__hip)
+
+
+def DQK_OF(kw):
+    return kw["DQK"]
+
+
+def DHV_OF(kw):
+    return kw["DHV"]
 
 
 def report_offenders(x, ref, name, rtol=2e-2, atol=2e-2):
@@ -569,11 +581,13 @@ def test_chunkwise_every_element_within_tolerance_of_the_rounding_emulation(kw, 
     |x - ref| <= 2e-2 + 2e-2 |ref|, no allowance.  The elements that miss this bound against the exact oracle in the
     other tests are therefore the 16-bit operand format's, not the kernels'.  The row normalisers are held to fp32
     summation accuracy first (a denominator whose terms nearly cancel cannot be more accurate than that in fp32, and
-    the whole row scales with it), then handed to the emulation.  Split path, every state stride."""
+    the whole row scales with it), then handed to the emulation.  Split and stream paths, every state stride."""
     import rounding_emulation as R
 
-    if not kernel_variant.startswith("split"):
-        pytest.skip("the emulation groups the products like the split path")
+    if kernel_variant.startswith("fused"):
+        pytest.skip("the emulation groups the products like the split and stream paths")
+    if kernel_variant.startswith("stream") and not (DQK_OF(kw) == 256 and DHV_OF(kw) % 512 == 0 and kw["S"] % 128 == 0):
+        pytest.skip("the stream path does not support this shape")
     stride = int(kernel_variant.split("-")[1])
     kw = dict(kw)
     B, NH, S, DQK, DHV = (kw.pop(n) for n in ("B", "NH", "S", "DQK", "DHV"))
@@ -599,7 +613,8 @@ def test_chunkwise_every_element_within_tolerance_of_the_rounding_emulation(kw, 
     track_n = not (siging and not normalize)
     _, qb, kb, vb, ib, fb, c0f, n0f, m0f = X._prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
     n_kernel = torch.empty(B, NH, S, dtype=torch.float32, device=DEV)
-    X._fw_launch(qb, kb, vb, ib, fb, c0f, n0f, m0f, 1e-6, siging, normalize, False, False, _lib.PATH_SPLIT, stride,
+    path = _lib.PATH_STREAM if kernel_variant.startswith("stream") else _lib.PATH_SPLIT
+    X._fw_launch(qb, kb, vb, ib, fb, c0f, n0f, m0f, 1e-6, siging, normalize, False, False, path, stride,
                  n_out=n_kernel)
     rnd = R.rounder(dtype)
     results = []
@@ -697,7 +712,7 @@ def test_recompute_states_in_bw_matches_kept_states(kw, kernel_variant):
     H_keep, g_keep, held_keep = run(False)
     H_rec, g_rec, held_rec = run(True)
     assert torch.equal(H_keep, H_rec)
-    exact = kernel_variant.startswith("split") and not last
+    exact = not kernel_variant.startswith("fused") and not last
     for name, a, b in zip(["dQ", "dK", "dV", "dI", "dF", "dC0"], g_rec, g_keep):
         if exact:
             assert torch.equal(a, b), f"{name} differs from the kept-states call"
