@@ -85,6 +85,14 @@ const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, h
     return mlstm::launch_stream_hv(a, BH, is_dv, st);
   return mlstm::launch_par_hv(a, BH, is_dv, st);
 }
+// dQ / dK launch: the streaming kernel under the same rule
+const char* launch_qk(int path, const mlstm::ParQkArgs& a, int BH, hipStream_t st) {
+  if (path == MLSTM_PATH_STREAM && !mlstm::stream_qk_supported(a))
+    return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 without head norm only";
+  if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::stream_qk_supported(a))
+    return mlstm::launch_stream_qk(a, BH, st);
+  return mlstm::launch_par_qk_pair(a, BH, st);
+}
 const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {
   if (B <= 0 || NH <= 0 || S <= 0) return "B, NH and S must be positive";
   if (DHQK <= 0 || DHHV <= 0 || DHQK % 64 != 0 || DHHV % 64 != 0) return "DHQK and DHHV must be positive multiples of 64";
@@ -499,7 +507,7 @@ int mlstm_hip_chunkwise_bw(const void* q, const void* k, const void* v, const vo
   pq.states2 = bws.dcstates; pq.Out2 = (uint16_t*)dK; pq.rowdot2 = bws.kdk;
   {
     ProfileScope ps("par_dqdk", st);
-    if (const char* e = mlstm::launch_par_qk_pair(pq, BH, st)) return fail(e);
+    if (const char* e = launch_qk(path, pq, BH, st)) return fail(e);
   }
   if (check_launch("par_qk dQ+dK")) return 1;
 
