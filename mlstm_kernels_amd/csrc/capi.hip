@@ -89,8 +89,8 @@ const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, h
 const char* launch_qk(int path, const mlstm::ParQkArgs& a, int BH, hipStream_t st) {
   if (path == MLSTM_PATH_STREAM && !mlstm::stream_qk_supported(a))
     return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 without head norm only";
-  if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::stream_qk_supported(a))
-    return mlstm::launch_stream_qk(a, BH, st);
+  // (MLSTM_PATH_AUTO keeps the tiled pair kernel: it is the faster one of the two as measured today)
+  if (path == MLSTM_PATH_STREAM && mlstm::stream_qk_supported(a)) return mlstm::launch_stream_qk(a, BH, st);
   return mlstm::launch_par_qk_pair(a, BH, st);
 }
 const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {

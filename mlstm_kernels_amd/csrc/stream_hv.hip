@@ -70,24 +70,6 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 }  // namespace
 
-#ifdef HV_EXP_TIMING
-__device__ unsigned long long g_hv_dbg[32];
-#define HV_SYNC()                                                     \
-  {                                                                   \
-    const unsigned long long t0_ = __builtin_amdgcn_s_memrealtime();  \
-    __syncthreads();                                                  \
-    const unsigned long long t1_ = __builtin_amdgcn_s_memrealtime();  \
-    dbg_wait += t1_ - t0_;                                            \
-    dbg_n += 1;                                                       \
-  }
-#define HV_TB(k) unsigned long long treg_##k = 0; if ((k) == HV_T_REGION) treg_##k = __builtin_amdgcn_s_memrealtime();
-#define HV_TE(k) if ((k) == HV_T_REGION) { dbg_reg += __builtin_amdgcn_s_memrealtime() - treg_##k; dbg_regn += 1; }
-#else
-#define HV_SYNC() __syncthreads()
-#define HV_TB(k)
-#define HV_TE(k)
-#endif
-
 template <bool IS_DV, bool F16>
 __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items, int n_rounds) {
   constexpr int DHQK = 256;
@@ -114,11 +96,6 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
   float* const mcv = denq + 128;               // [128] forward: combined stabiliser of the item's positions
   constexpr uint32_t kRing0Off = 128 * QS * 2, kRing1Off = kRing0Off + (SLOT + 128 * PSS) * 2;
 
-#ifdef HV_EXP_TIMING
-  unsigned long long dbg_wait = 0, dbg_n = 0;
-  unsigned long long dbg_reg = 0, dbg_regn = 0;
-  const unsigned long long dbg_start = __builtin_amdgcn_s_memrealtime();
-#endif
   const int lane = threadIdx.x & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int G = gridDim.x;
@@ -130,9 +107,9 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
 
   if (wave_all >= 8) {
     // =========================================================================================== producer waves
-    // Load step L (counted over all items of this workgroup) uses register set L & 1.  Handling it means: pass barrier
-    // L - 3 (the consumers are done with slab L - 4, whose ring slot slab L - 2 goes into), write slab L - 2 from the
-    // register set to LDS, request slab L into the set.  The destination in LDS travels with the data: byte offset of
+    // Load step L (counted over all items of this workgroup) uses register set L % 3.  Handling it means: pass barrier
+    // L - 4 (the consumers are done with slab L - 5, whose ring slot slab L - 3 goes into), write slab L - 3 from the
+    // register set to LDS, request slab L into the set: three slabs are on their way at any time.  The destination in LDS travels with the data: byte offset of
     // the thread's first piece | slab kind << 20 (0 fragment-order rows, 1 state fragments, 3 value rows) | gate-vector
     // flag << 22; the thread's other seven pieces lie a fixed distance apart.
     const int p = (wave_all - 8) * 64 + lane;  // 0 .. 255: every thread moves eight 16-byte pieces of every slab
@@ -142,77 +119,100 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
     const char* const St_b = (const char*)a.states;
     const float* const ov_src = IS_DV ? a.g.u : a.g.w;
     const float* const rho_src = (IS_DV && a.use_nrow) ? a.nrow : ov_src;
-    uint4 fd[2][8];
-    uint32_t fw[2];
-    float fa[2][2];
+    // three register sets, named by a pasted literal
+    u32x4 fd0[8], fd1[8], fd2[8];
+    uint32_t fw0 = 0, fw1 = 0, fw2 = 0;
+    float fa0[2], fa1[2], fa2[2];
     int L = 0;
 #define HV_STORE(E)                                                                                                  \
   {                                                                                                                  \
-    const uint32_t w_ = fw[E];                                                                                       \
+    const uint32_t w_ = fw##E;                                                                                       \
     const uint32_t kind_ = (uint32_t)__builtin_amdgcn_readfirstlane((int)((w_ >> 20) & 3));                          \
+    const bool whole_ = __builtin_amdgcn_readfirstlane((int)((w_ >> 23) & 1)) == 0;                                  \
     const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
     const uint32_t half_ = kind_ == 0 ? 16u : 8u;                                                                    \
     const uint32_t step_ = kind_ == 0 ? 8 * QS * 2 : (kind_ == 1 ? 4096 : 4 * VS * 2);                               \
-    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) {                                                               \
-      *(uint2*)(smem_raw + d0_ + i_ * step_) = make_uint2(fd[E][i_].x, fd[E][i_].y);                                 \
-      *(uint2*)(smem_raw + d0_ + i_ * step_ + half_) = make_uint2(fd[E][i_].z, fd[E][i_].w);                         \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                               \
+      *(uint2*)(smem_raw + d0_ + i_ * step_) = make_uint2(fd##E[i_][0], fd##E[i_][1]);                               \
+      *(uint2*)(smem_raw + d0_ + i_ * step_ + half_) = make_uint2(fd##E[i_][2], fd##E[i_][3]);                       \
+    }                                                                                                                \
+    if (whole_) {                                                                                                    \
+      _Pragma("unroll") for (int i_ = 4; i_ < 8; ++i_) {                                                             \
+        *(uint2*)(smem_raw + d0_ + i_ * step_) = make_uint2(fd##E[i_][0], fd##E[i_][1]);                             \
+        *(uint2*)(smem_raw + d0_ + i_ * step_ + half_) = make_uint2(fd##E[i_][2], fd##E[i_][3]);                     \
+      }                                                                                                              \
     }                                                                                                                \
     if (__builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 64) {                                           \
-      ovec[p] = fa[E][0] * kLog2e;                                                                                   \
-      if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa[E][1] + a.eps) : 1.f;                                              \
+      ovec[p] = fa##E[0] * kLog2e;                                                                                   \
+      if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa##E[1] + a.eps) : 1.f;                                              \
     }                                                                                                                \
   }
     // base_: (batch, head) base of the operand; g0_: byte offset of the thread's first piece, gs_: distance between
     // its pieces; gi_: index of the gate-vector entry that rides along (stored only with the flag set; the other
-    // slabs request an entry all the same so that every step issues the same loads)
-#ifdef HV_EXP_NOLOAD
-#define HV_EXP_LOADS(E, base_, g0_, gs_, gi_)                                                                        \
+    // slabs request an entry all the same so that every step issues the same loads); NP_: pieces per thread (8, or 4
+    // for the half-size slabs of the resident rows, flagged by bit 23 of the destination word)
+#define HV_PROC(E, NP_, base_, g0_, gs_, dstw_, gi_)                                                                 \
   {                                                                                                                  \
-    fa[E][0] = (float)(g0_); fa[E][1] = 1.f;                                                                         \
-    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) fd[E][i_] = make_uint4((g0_) + i_ * (gs_), 0, 0, 0);            \
-    (void)(base_); (void)(gi_);                                                                                      \
-  }
-#else
-#define HV_EXP_LOADS(E, base_, g0_, gs_, gi_)                                                                        \
-  {                                                                                                                  \
-    fa[E][0] = ov_src[gi_];                                                                                          \
-    fa[E][1] = rho_src[gi_];                                                                                         \
-    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) fd[E][i_] = *(const uint4*)((base_) + ((g0_) + i_ * (gs_)));    \
-  }
-#endif
-#define HV_PROC(E, base_, g0_, gs_, dstw_, gi_)                                                                      \
-  {                                                                                                                  \
-    if (L >= 3) HV_SYNC();                                                                                           \
-    HV_TB(6) if (L >= 2) HV_STORE(E) HV_TE(6)                                                                        \
-    HV_TB(7) HV_EXP_LOADS(E, base_, g0_, gs_, gi_) HV_TE(7)                                                          \
-    fw[E] = (dstw_);                                                                                                 \
+    if (L >= 4) __syncthreads();                                                                                           \
+    /* piece by piece: the old content of a register goes to LDS, then the register is requested anew, so that the */ \
+    /* LDS port and the vector-memory path of the CU work side by side instead of one after the other */             \
+    const uint32_t w_ = fw##E;                                                                                       \
+    const uint32_t kind_ = (uint32_t)__builtin_amdgcn_readfirstlane((int)((w_ >> 20) & 3));                          \
+    const bool whole_ = __builtin_amdgcn_readfirstlane((int)((w_ >> 23) & 1)) == 0;                                  \
+    const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
+    const uint32_t half_ = kind_ == 0 ? 16u : 8u;                                                                    \
+    const uint32_t step_ = kind_ == 0 ? 8 * QS * 2 : (kind_ == 1 ? 4096 : 4 * VS * 2);                               \
+    const bool st_ = L >= 3;                                                                                         \
+    if (st_ && __builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 64) {                                    \
+      ovec[p] = fa##E[0] * kLog2e;                                                                                   \
+      if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa##E[1] + a.eps) : 1.f;                                              \
+    }                                                                                                                \
+    fa##E[0] = ov_src[gi_];                                                                                          \
+    fa##E[1] = rho_src[gi_];                                                                                         \
+    _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) {                                                               \
+      if (st_ && (i_ < 4 || whole_)) {                                                                               \
+        *(uint2*)(smem_raw + d0_ + i_ * step_) = make_uint2(fd##E[i_][0], fd##E[i_][1]);                             \
+        *(uint2*)(smem_raw + d0_ + i_ * step_ + half_) = make_uint2(fd##E[i_][2], fd##E[i_][3]);                     \
+      }                                                                                                              \
+      if (i_ < (NP_)) fd##E[i_] = *(const u32x4*)((base_) + ((g0_) + i_ * (gs_)));                                             \
+    }                                                                                                                \
+    fw##E = (dstw_) | ((NP_) == 4 ? 1u << 23 : 0u);                                                                  \
     ++L;                                                                                                             \
   }
     HvItem it;
     for (int rd = 0; rd < n_rounds; ++rd) {
       if (!hv_decode<IS_DV>(it, rd, vid, G, n_items, NC, NCH, stride)) continue;
+      // An item has 12 + 6 s steps, a multiple of three: the register set of every step is a literal.
       const uint32_t pl = (uint32_t)opaque(p);
       const uint32_t row = pl >> 5, pc = pl & 31;  // rows of 512 bytes: 32 pieces per row, 8 rows per sweep
       const size_t gown = (size_t)it.bh * Sp + (size_t)it.c * kChunk + (pl & 63);
       // fragment-order destination of piece pc inside a row (see store_perm16)
       const uint32_t permo = (pc >> 1) * 32 + 8 * (pc & 1);
       {
-        // ---- resident rows
+        // ---- resident rows, 32 per step (half-size slabs: four steps for the consumers' epilogue of the previous
+        // item, and a step count per item that is a multiple of three)
         const char* const base = Xn_b + (size_t)it.bh * S * DHQK * 2;
         const uint32_t g0 = ((uint32_t)(it.c * kChunk) + row) * (DHQK * 2) + pc * 16;
         const uint32_t d0 = row * (QS * 2) + permo;
-        HV_PROC(0, base, g0, 8 * DHQK * 2, d0, gown)
-        HV_PROC(1, base, g0 + 64 * DHQK * 2, 8 * DHQK * 2, d0 + 64 * QS * 2, gown)
+        HV_PROC(0, 4, base, g0, 8 * DHQK * 2, d0, gown)
+        HV_PROC(1, 4, base, g0 + 32 * DHQK * 2, 8 * DHQK * 2, d0 + 32 * QS * 2, gown)
+        HV_PROC(2, 4, base, g0 + 64 * DHQK * 2, 8 * DHQK * 2, d0 + 64 * QS * 2, gown)
+        HV_PROC(0, 4, base, g0 + 96 * DHQK * 2, 8 * DHQK * 2, d0 + 96 * QS * 2, gown)
       }
       {
         // ---- state fragments: slab si holds contraction steps 2 si, 2 si + 1 of the sixteen 32-column blocks
         const char* const base = St_b + ((size_t)it.bh * NCS + it.slot) * (size_t)(DHHV / 32) * ND * 1024;
         const uint32_t f0 = pl >> 6;  // fragment of the first piece inside the slab: block f0 / 2, contraction step f0 % 2
         const uint32_t g0 = (((uint32_t)it.ch * 16 + (f0 >> 1)) * ND + (f0 & 1)) * 1024 + (pl & 63) * 16;
-        for (int si = 0; si < 8; si += 2) {
-          HV_PROC(0, base, g0 + si * 2048, 2 * ND * 1024, (kRing0Off + pl * 16) | (1u << 20), gown)
-          HV_PROC(1, base, g0 + (si + 1) * 2048, 2 * ND * 1024, (kRing1Off + pl * 16) | (1u << 20), gown)
-        }
+        const uint32_t r0 = (kRing0Off + pl * 16) | (1u << 20), r1 = (kRing1Off + pl * 16) | (1u << 20);
+        HV_PROC(1, 8, base, g0, 2 * ND * 1024, r0, gown)
+        HV_PROC(2, 8, base, g0 + 1 * 2048, 2 * ND * 1024, r1, gown)
+        HV_PROC(0, 8, base, g0 + 2 * 2048, 2 * ND * 1024, r0, gown)
+        HV_PROC(1, 8, base, g0 + 3 * 2048, 2 * ND * 1024, r1, gown)
+        HV_PROC(2, 8, base, g0 + 4 * 2048, 2 * ND * 1024, r0, gown)
+        HV_PROC(0, 8, base, g0 + 5 * 2048, 2 * ND * 1024, r1, gown)
+        HV_PROC(1, 8, base, g0 + 6 * 2048, 2 * ND * 1024, r0, gown)
+        HV_PROC(2, 8, base, g0 + 7 * 2048, 2 * ND * 1024, r1, gown)
       }
       {
         const char* const kbase = Xo_b + (size_t)it.bh * S * DHQK * 2;
@@ -226,37 +226,33 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
           const size_t gi = (size_t)it.bh * Sp + (size_t)sc * kChunk + (pl & 63);
           const uint32_t vg = (t0 + vrow) * (uint32_t)(DHHV * 2) + (uint32_t)it.ch * 1024 + vpc * 16;
           const uint32_t vgs = 4 * (uint32_t)DHHV * 2, vg32 = 32 * (uint32_t)DHHV * 2;
-          // first half: scores -> set 0 / slot 0, value rows -> set 1 / slot 1 and set 0 / slot 0
-          HV_PROC(0, kbase, (t0 + row) * (DHQK * 2) + pc * 16, 8 * DHQK * 2, (kRing0Off + kd) | (1u << 22), gi)
-          HV_PROC(1, vbase, vg, vgs, kRing1Off + vd, gown)
-          HV_PROC(0, vbase, vg + vg32, vgs, kRing0Off + vd, gown)
+          // first half: scores -> slot 0, value rows -> slot 1 and slot 0
+          HV_PROC(0, 8, kbase, (t0 + row) * (DHQK * 2) + pc * 16, 8 * DHQK * 2, (kRing0Off + kd) | (1u << 22), gi)
+          HV_PROC(1, 8, vbase, vg, vgs, kRing1Off + vd, gown)
+          HV_PROC(2, 8, vbase, vg + vg32, vgs, kRing0Off + vd, gown)
           // second half: the other way round
-          HV_PROC(1, kbase, (t0 + 64 + row) * (DHQK * 2) + pc * 16, 8 * DHQK * 2, (kRing1Off + kd) | (1u << 22), gi + 64)
-          HV_PROC(0, vbase, vg + 2 * vg32, vgs, kRing0Off + vd, gown)
-          HV_PROC(1, vbase, vg + 3 * vg32, vgs, kRing1Off + vd, gown)
+          HV_PROC(0, 8, kbase, (t0 + 64 + row) * (DHQK * 2) + pc * 16, 8 * DHQK * 2, (kRing1Off + kd) | (1u << 22), gi + 64)
+          HV_PROC(1, 8, vbase, vg + 2 * vg32, vgs, kRing0Off + vd, gown)
+          HV_PROC(2, 8, vbase, vg + 3 * vg32, vgs, kRing1Off + vd, gown)
         }
       }
     }
-    // ---- drain: the last two slabs go to LDS, then the barriers of the consumers' last steps and of the final epilogue
+    // ---- drain: the last three slabs go to LDS, then the barriers of the consumers' last steps and of the final epilogue
     if (L > 0) {
-      if (L >= 3) HV_SYNC();
+      if (L >= 4) __syncthreads();
       HV_STORE(0)
-      HV_SYNC();
+      __syncthreads();
       HV_STORE(1)
-      HV_SYNC();
-      HV_SYNC();
-      HV_SYNC();
+      __syncthreads();
+      HV_STORE(2)
+      __syncthreads();
+      __syncthreads();
+      __syncthreads();
     }
 #undef HV_PROC
-#undef HV_EXP_LOADS
 #undef HV_STORE
   } else {
     // =========================================================================================== consumer waves
-#ifdef HV_EXP_NOMFMA
-#define HV_MFMA(C_, A_, B_) { (C_)[0] += __uint_as_float((A_).w[0] ^ (B_).w[0]); }
-#else
-#define HV_MFMA(C_, A_, B_) mfma32<F16>(C_, A_, B_)
-#endif
     const int wave = wave_all;
     const int tid = wave * 64 + lane;
     const int pi = wave & 1, ci = wave >> 1;  // output role: positions 64 pi .., value columns 128 ci .. of the item
@@ -310,8 +306,7 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
       // positions, then the other 32 in two rounds of 64 columns: the second step has less LDS to stage through), the
       // per-item vectors are requested
       float csr[2], nv, cs0r = 0.f, mcr = 0.f, np0 = 0.f, np1 = 0.f, np2 = 0.f;
-      HV_SYNC();
-      HV_TB(5)
+      __syncthreads();
       if (have_prev) HV_EPILOGUE(0, 0, 4, Ring0 + wave * (32 * 136))
       {
         const int r = opaque(lane) & 31;
@@ -344,17 +339,15 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
           }
         }
       }
-      HV_TE(5)
-      HV_SYNC();
-      if (have_prev) {
-        HV_EPILOGUE(1, 0, 2, Ps + wave * (32 * 72))
-        HV_EPILOGUE(1, 2, 2, Ps + wave * (32 * 72))
-      }
+      __syncthreads();
+      if (have_prev) HV_EPILOGUE(1, 0, 4, Ring0 + wave * (32 * 136))
+      __syncthreads();
       if (!IS_DV && tid < DHQK) nperm[perm16(tid)] = (np0 + np1) + np2;
+      __syncthreads();
       // ---- inter-chunk product: Out^T = State^T Xn^T, two contraction steps per slab
 #pragma unroll
       for (int si = 0; si < 8; ++si) {
-        HV_SYNC();
+        __syncthreads();
         if (!IS_DV) {
           if (si == 0) {
             // forward: q_t . n_prev for the denominators (four threads per position), while the resident rows are
@@ -389,7 +382,6 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
 #pragma unroll
               for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.f;
         }
-        HV_TB(1)
         const int le = opaque(lane);
         const int r = le & 31, h = le >> 5;
         const uint16_t* const slab = (si & 1) ? Ring1 : Ring0;
@@ -404,9 +396,8 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
 #pragma unroll
           for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) HV_MFMA(acc[mb][nb], A[mb], B[nb]);
+            for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[mb][nb], A[mb], B[nb]);
         }
-        HV_TE(1)
       }
       // (kept apart from the matrix instructions around it: interleaved with them the products land in fresh
       // registers, a second copy of an accumulator tile the register file has no room for)
@@ -432,9 +423,8 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
           // scores of position block pb against source block kb of this half
 #pragma unroll
           for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-          HV_SYNC();
+          __syncthreads();
           {
-            HV_TB(2)
             const int le = opaque(lane);
             const int r = le & 31, h = le >> 5;
             // blocks of the own chunk that the causal mask empties are not multiplied (their rows stay zero)
@@ -445,11 +435,9 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
                 Frag A, B;
                 A.u = *(const uint4*)(kslab + (32 * kb + r) * QS + 16 * ds + 8 * h);
                 B.u = *(const uint4*)(Ns + (32 * pb + r) * QS + 16 * ds + 8 * h);
-                HV_MFMA(sacc, A, B);
+                mfma32<F16>(sacc, A, B);
               }
             }
-            HV_TE(2)
-            HV_TB(3)
             // gate, mask, round and write P as Ps[n][o]; forward: fp32 row sums over the own chunk's positions
             const int n = 32 * pb + r;  // position inside the chunk
             float rsum = 0.f;
@@ -481,13 +469,11 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
               const float tot = rsum + __shfl_xor(rsum, 32);
               if (h == 0) rows[(2 * kh + kb) * 128 + n] = tot;  // blocks above the diagonal publish zero
             }
-            HV_TE(3)
           }
           // Out^T += Xw^T P over the 64 source positions of the half: two slabs of 32
 #pragma unroll
           for (int vi = 0; vi < 2; ++vi) {
-            HV_SYNC();
-            HV_TB(4)
+            __syncthreads();
             const int le = opaque(lane);
             const int r = le & 31, h = le >> 5;
             const int q16 = (le >> 4) & 1, i16 = le & 15;
@@ -508,9 +494,8 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
 #pragma unroll
               for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb) HV_MFMA(acc[mb][nb], A[mb], B[nb]);
+                for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[mb][nb], A[mb], B[nb]);
             }
-            HV_TE(4)
             // ---- forward: denominators, once all row sums of the own chunk are there (it is the last source chunk)
             if (!IS_DV && own && kh == 1 && vi == 1) {
               const int td = opaque(tid);
@@ -542,25 +527,13 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
       have_prev = true;
     }
     if (have_prev) {
-      HV_SYNC();
+      __syncthreads();
       HV_EPILOGUE(0, 0, 4, Ring0 + wave * (32 * 136))
-      HV_SYNC();
-      HV_EPILOGUE(1, 0, 2, Ps + wave * (32 * 72))
-      HV_EPILOGUE(1, 2, 2, Ps + wave * (32 * 72))
+      __syncthreads();
+      HV_EPILOGUE(1, 0, 4, Ring0 + wave * (32 * 136))
     }
 #undef HV_EPILOGUE
-#undef HV_MFMA
   }
-#ifdef HV_EXP_TIMING
-  if (blockIdx.x == 0 && lane == 0 && (wave_all == 0 || wave_all == 8)) {
-    const int o = (wave_all == 8 ? 8 : 0) + (IS_DV ? 16 : 0);
-    g_hv_dbg[o] = dbg_wait;
-    g_hv_dbg[o + 1] = dbg_n;
-    g_hv_dbg[o + 2] = __builtin_amdgcn_s_memrealtime() - dbg_start;
-    g_hv_dbg[o + 4] = dbg_reg;
-    g_hv_dbg[o + 5] = dbg_regn;
-  }
-#endif
 }
 
 bool stream_hv_supported(const ParHvArgs& a) {
@@ -609,8 +582,3 @@ const char* launch_stream_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t
 
 }  // namespace mlstm
 
-#ifdef HV_EXP_TIMING
-extern "C" int mlstm_debug_read(unsigned long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(mlstm::g_hv_dbg), sizeof(unsigned long long) * 32);
-}
-#endif

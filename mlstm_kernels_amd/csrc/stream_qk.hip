@@ -57,23 +57,6 @@ constexpr float kQkLog2e = 1.4426950408889634f;
 
 }  // namespace
 
-#ifdef QK_EXP_TIMING
-__device__ unsigned long long g_qk_dbg[32];
-#define QK_SYNC()                                                     \
-  {                                                                   \
-    const unsigned long long t0_ = __builtin_amdgcn_s_memrealtime();  \
-    __syncthreads();                                                  \
-    const unsigned long long t1_ = __builtin_amdgcn_s_memrealtime();  \
-    dbg_wait += t1_ - t0_;                                            \
-    dbg_n += 1;                                                       \
-  }
-#define QK_TB(k) unsigned long long treg_##k = 0; if ((k) == QK_T_REGION) treg_##k = __builtin_amdgcn_s_memrealtime();
-#define QK_TE(k) if ((k) == QK_T_REGION) { dbg_reg += __builtin_amdgcn_s_memrealtime() - treg_##k; dbg_regn += 1; }
-#else
-#define QK_SYNC() __syncthreads()
-#define QK_TB(k)
-#define QK_TE(k)
-#endif
 template <bool F16>
 __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items, int n_rounds) {
   constexpr int DHQK = 256;
@@ -90,10 +73,6 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
   float* const orho = ovec + 128;                 // [128] dK: rho_t of the source chunk (dQ: ones)
   float* const red = orho + 128;                  // [4][128] row-dot partials of the previous item, per 64-row block
 
-#ifdef QK_EXP_TIMING
-  unsigned long long dbg_wait = 0, dbg_n = 0, dbg_reg = 0, dbg_regn = 0;
-  const unsigned long long dbg_start = __builtin_amdgcn_s_memrealtime();
-#endif
   const int lane = threadIdx.x & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int G = gridDim.x;
@@ -129,29 +108,29 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
   }
     // one step: bA_/gA_/sA_ base, first byte offset and piece distance of pieces 0..3, bB_/gB_/sB_ of pieces 4..7
     // (a row slab has two sources); dst_ destination word without the slot; gi_ gate-vector index that rides along
-#ifdef QK_EXP_NOLOAD
-#define QK_LOADS(E, bA_, gA_, sA_, bB_, gB_, sB_, gi_)                                                               \
-  {                                                                                                                  \
-    fa##E[0] = (float)(gA_); fa##E[1] = 1.f; (void)(bA_); (void)(bB_); (void)(gi_);                                   \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd##E[i_] = u32x4{(gA_) + i_ * (sA_), 0u, 0u, 0u};              \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd##E[4 + i_] = u32x4{(gB_) + i_ * (sB_), 0u, 0u, 0u};          \
-  }
-#else
-#define QK_LOADS(E, bA_, gA_, sA_, bB_, gB_, sB_, gi_)                                                               \
-  {                                                                                                                  \
-    fa##E[0] = ov_src[gi_];                                                                                          \
-    fa##E[1] = rho_src[gi_];                                                                                         \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd##E[i_] = *(const u32x4*)((bA_) + ((gA_) + i_ * (sA_)));      \
-    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) fd##E[4 + i_] = *(const u32x4*)((bB_) + ((gB_) + i_ * (sB_)));  \
-  }
-#endif
 #define QK_PROC(E, bA_, gA_, sA_, bB_, gB_, sB_, dst_, gi_)                                                          \
   {                                                                                                                  \
-    if (L >= 3) QK_SYNC();                                                                                     \
-    QK_TB(6) if (L >= 2) QK_STORE(E) QK_TE(6)                                                                        \
-    QK_TB(7)                                                                                                         \
-    QK_LOADS(E, bA_, gA_, sA_, bB_, gB_, sB_, gi_)                                                                   \
-    QK_TE(7)                                                                                                         \
+    if (L >= 3) __syncthreads();                                                                                           \
+    /* piece by piece: the old content of a register goes to LDS, then the register is requested anew, so that the */ \
+    /* LDS port and the vector-memory path of the CU work side by side instead of one after the other */             \
+    const uint32_t w_ = fw##E;                                                                                       \
+    const uint32_t step_ = __builtin_amdgcn_readfirstlane((int)((w_ >> 20) & 1)) ? 4608u : 4096u;                    \
+    const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
+    const bool st_ = L >= 2;                                                                                         \
+    if (st_ && __builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 128) {                                   \
+      ovec[p] = fa##E[0] * kQkLog2e;                                                                                 \
+      orho[p] = __builtin_amdgcn_readfirstlane((int)((w_ >> 23) & 1)) ? 1.f / (fa##E[1] + a.eps) : 1.f;              \
+    }                                                                                                                \
+    fa##E[0] = ov_src[gi_];                                                                                          \
+    fa##E[1] = rho_src[gi_];                                                                                         \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                               \
+      if (st_) *(u32x4*)(smem_raw + d0_ + i_ * step_) = fd##E[i_];                                                   \
+      fd##E[i_] = *(const u32x4*)((bA_) + ((gA_) + i_ * (sA_)));                                                     \
+    }                                                                                                                \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) {                                                               \
+      if (st_) *(u32x4*)(smem_raw + d0_ + (4 + i_) * step_) = fd##E[4 + i_];                                         \
+      fd##E[4 + i_] = *(const u32x4*)((bB_) + ((gB_) + i_ * (sB_)));                                                 \
+    }                                                                                                                \
     fw##E = (dst_) + ring_slot * (SLOT * 2);                                                                         \
     ring_slot = ring_slot == 2 ? 0 : ring_slot + 1;                                                                  \
     ++L;                                                                                                             \
@@ -204,12 +183,12 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
     }
     // ---- drain: the last two slabs go to LDS, then the barriers of the consumers' last steps and of the final row dots
     if (L > 0) {
-      if (L >= 3) QK_SYNC();
+      if (L >= 3) __syncthreads();
       QK_STORE(0)
-      QK_SYNC();
+      __syncthreads();
       QK_STORE(1)
-      QK_SYNC();
-      QK_SYNC();
+      __syncthreads();
+      __syncthreads();
     }
 #undef QK_PROC
 #undef QK_STORE
@@ -278,10 +257,9 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
       // causal mask empties the blocks with o > n (dQ) or o < n (dK); a wave whose two blocks are both empty skips the
       // multiplications (its rows of P stay zero).
 #define QK_XSTEP(LIVE_)                                                                                              \
-  QK_SYNC();                                                                                                   \
+  __syncthreads();                                                                                                   \
   const uint16_t* const Xn = Ring + next_slot() * SLOT;                                                              \
   {                                                                                                                  \
-    QK_TB(1)                                                                                                         \
     const uint16_t* const Xo = Xn + 128 * XS;                                                                        \
     const int le = opaque(lane);                                                                                     \
     const int r = le & 31, h = le >> 5;                                                                              \
@@ -294,13 +272,11 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
         _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) mfma32<F16>(sacc[kk], A[kk], B);                            \
       }                                                                                                              \
     }                                                                                                                \
-    QK_TE(1)                                                                                                         \
   }
       // Gate the score blocks: P[o][n] = scores * exp(u_t - w_j + G) / sqrt(DHQK) * rho_t (own chunk: masked), stored
       // as Ps[n][o]; sc_: source chunk, OWN_: it is the own one
 #define QK_GATE(sc_, OWN_)                                                                                           \
   {                                                                                                                  \
-    QK_TB(3)                                                                                                         \
     float gs = 0.f; /* decay between the two chunks */                                                               \
     for (int x = (dk ? c : (sc_)); x < (dk ? (sc_) : c); ++x) gs += graw[x];                                         \
     const float sgn = dk ? -1.f : 1.f;                                                                               \
@@ -323,15 +299,13 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
       }                                                                                                              \
       *(uint2*)(Ps + n * PS + o0) = make_uint2(pack2<F16>(pv[0], pv[1]), pack2<F16>(pv[2], pv[3]));                  \
     }                                                                                                                \
-    QK_TE(3)                                                                                                         \
   }
       // Out^T += Z^T P over the 128 source positions, 64 per slab; LAST_: the x rows of the row dots are requested
       // with the first slab
 #define QK_PASS2(LAST_)                                                                                              \
   _Pragma("unroll") for (int zs = 0; zs < 2; ++zs) {                                                                 \
-    QK_SYNC();                                                                                                 \
+    __syncthreads();                                                                                                 \
     const uint16_t* const Zs = Ring + next_slot() * SLOT;                                                            \
-    QK_TB(4)                                                                                                         \
     const int le = opaque(lane);                                                                                     \
     const int r = le & 31, h = le >> 5;                                                                              \
     const int q16 = (le >> 4) & 1, i16 = le & 15;                                                                    \
@@ -354,7 +328,6 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
       _Pragma("unroll") for (int mb = 0; mb < 2; ++mb) _Pragma("unroll") for (int nb = 0; nb < 2; ++nb)              \
         mfma32<F16>(acc[mb][nb], A[mb], B[nb]);                                                                      \
     }                                                                                                                \
-    QK_TE(4)                                                                                                         \
   }
 #define QK_ZERO_SCORES                                                                                               \
   _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) _Pragma("unroll") for (int i = 0; i < 16; ++i) sacc[kk][i] = 0.f;
@@ -370,9 +343,8 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
           // Out^T += State Xn^T.  The stored fragments (made for a contraction over the head dimension) are read with
           // the transposing LDS read: lane i16 of a 16-lane block addresses value column k0 + i16 / 4 and the 4
           // consecutive head-dim rows n0 + 4 (i16 % 4) .. + 3
-          QK_SYNC();
+          __syncthreads();
           const uint16_t* const Cf = Ring + next_slot() * SLOT;
-          QK_TB(2)
           const int le = opaque(lane);
           const int r = le & 31, h = le >> 5;
           const int q16 = (le >> 4) & 1, i16 = le & 15;
@@ -403,7 +375,6 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[mb][nb], A[mb], B[nb]);
             }
-          QK_TE(2)
         }
         // column scale of the inter-chunk part (kept apart from the matrix instructions around it)
         __builtin_amdgcn_sched_barrier(0);
@@ -433,7 +404,6 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
         // ---- row dots sum_d x[n][d] * Out[n][d] from the fp32 accumulators (they feed a suffix sum over the whole
         // sequence, where the rounding noise of 16-bit outputs would add up), and the output rows, rounded, straight
         // from the accumulators: 16 contiguous bytes per row and lane pair
-        QK_TB(5)
         const int le = opaque(lane);
         const int r = le & 31, h = le >> 5;
         uint16_t* const Og = (dk ? a.Out2 : a.Out) + ((size_t)bh * S + (size_t)c * kChunk) * DHQK;
@@ -456,26 +426,15 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
           part += __shfl_xor(part, 32);
           if (h == 0) red[di * 128 + 64 * ni + 32 * nb + r] = part;
         }
-        QK_TE(5)
       }
       prev = it;
       have_prev = true;
     }
     if (have_prev) {
-      QK_SYNC();
+      __syncthreads();
       finish_rowdots();
     }
   }
-#ifdef QK_EXP_TIMING
-  if (blockIdx.x == 0 && lane == 0 && (wave_all == 0 || wave_all == 8)) {
-    const int o = (wave_all == 8 ? 8 : 0);
-    g_qk_dbg[o] = dbg_wait;
-    g_qk_dbg[o + 1] = dbg_n;
-    g_qk_dbg[o + 2] = __builtin_amdgcn_s_memrealtime() - dbg_start;
-    g_qk_dbg[o + 4] = dbg_reg;
-    g_qk_dbg[o + 5] = dbg_regn;
-  }
-#endif
 }
 
 bool stream_qk_supported(const ParQkArgs& a) { return a.DHQK == 256 && a.DHHV % 128 == 0 && a.S % kChunk == 0; }
@@ -522,8 +481,3 @@ const char* launch_stream_qk(const ParQkArgs& a, int BH, hipStream_t stream) {
 
 }  // namespace mlstm
 
-#ifdef QK_EXP_TIMING
-extern "C" int mlstm_debug_read(unsigned long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(mlstm::g_qk_dbg), sizeof(unsigned long long) * 32);
-}
-#endif
