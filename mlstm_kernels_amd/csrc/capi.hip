@@ -294,6 +294,10 @@ int chunkwise_fw_impl(const char* who, const void* q, const void* k, const void*
   sa.backward = 0;
   sa.stride = stride;
   sa.f16 = f16;
+  // Which chunks still weigh in the last state is read off the decay factors, which presumes inputs of comparable
+  // scale in every chunk: true for the exponential gate (its stabiliser rescales them), not for the sigmoid gate,
+  // whose late positions may all be closed while early chunks dominate the state.
+  sa.all_remainder = sig;
   {
     ProfileScope ps("scan_fw", st);
     // The head + remainder split of the value operand only serves the fp32 last state (1e-5 instead of 1.5e-3

@@ -26,6 +26,9 @@ struct ScanArgs {
   int backward;
   int stride;             // a chunk state is kept every `stride` chunks
   int f16;                // X, Y and the state fragments are float16 instead of bfloat16
+  int all_remainder;      // forward, last state returned: every chunk carries the remainder of the value operand (the
+                          // sigmoid input gate has no stabiliser, so the decay factors alone do not say which chunks
+                          // still weigh in the last state)
   int part;               // set by the launcher: 0 whole sequence; 1 / 2 the two launches of a forward scan that
                           // returns the last state (before / from the first chunk that carries the remainder)
 };

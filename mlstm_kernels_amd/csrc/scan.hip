@@ -203,7 +203,7 @@ __global__ __launch_bounds__(64 * (RT / 64) * (WT / WCOLS))
   // c_lo = first chunk that carries the remainder of the value operand
   int c_lo = 0;
   if constexpr (HILO) {
-    if (!a.backward) c_lo = first_remainder_chunk(a.gbar + (size_t)bh * NC, NC, lane);
+    if (!a.backward) c_lo = a.all_remainder ? 0 : first_remainder_chunk(a.gbar + (size_t)bh * NC, NC, lane);
   }
   // part 2 of a forward scan in two launches: the chunks from c_lo on, continuing from the state the first launch left
   // in final_out / n_final (loaded above)
@@ -641,7 +641,7 @@ __global__ __launch_bounds__(128 * (RT / 64) * (WT / 32)) void scan_roles_kernel
   const size_t Sp = (size_t)NC * kChunk;
   // part 1 of a forward scan in two launches: only the chunks before the first one that carries the remainder of the
   // value operand; the state reached there is handed over in final_out / n_final
-  const int n_run = a.part == 1 ? first_remainder_chunk(a.gbar + (size_t)bh * NC, NC, lane) : NC;
+  const int n_run = a.part == 1 ? (a.all_remainder ? 0 : first_remainder_chunk(a.gbar + (size_t)bh * NC, NC, lane)) : NC;
   const int total = n_run * NP;
   const int c_first = a.backward ? NC - 1 : 0, c_step = a.backward ? -1 : 1;
 

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
   float* const rows = (float*)(Ring1 + SLOT);  // [4][128] partial row sums of the own chunk's scores (forward)
   float* const inv = rows + 4 * 128;           // [128] forward: 1 / (row normaliser + eps)
   float* const nperm = inv + 128;              // [DHQK] forward: n before the chunk, fragment order
-  float* const ovec = nperm + DHQK;            // [64] gate vector of the source half times log2(e): w_j (forward) / u_t (dV)
+  float* const ovec = nperm + DHQK;            // [64] gate vector of the source half: w_j (forward) / u_t (dV)
   float* const orho = ovec + 64;               // [64] dV: rho_t of the source half
   float* const denq = orho + 64;               // [128] forward: bbar_t / sqrt(d) * (q_t . n_prev), the inter-chunk part of the denominator
   float* const mcv = denq + 128;               // [128] forward: combined stabiliser of the item's positions
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
       }                                                                                                              \
     }                                                                                                                \
     if (__builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 64) {                                           \
-      ovec[p] = fa##E[0] * kLog2e;                                                                                   \
+      ovec[p] = fa##E[0];                                                                                   \
       if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa##E[1] + a.eps) : 1.f;                                              \
     }                                                                                                                \
   }
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
     const uint32_t step_ = kind_ == 0 ? 8 * QS * 2 : (kind_ == 1 ? 4096 : 4 * VS * 2);                               \
     const bool st_ = L >= 3;                                                                                         \
     if (st_ && __builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 64) {                                    \
-      ovec[p] = fa##E[0] * kLog2e;                                                                                   \
+      ovec[p] = fa##E[0];                                                                                   \
       if (IS_DV) orho[p] = a.use_nrow ? 1.f / (fa##E[1] + a.eps) : 1.f;                                              \
     }                                                                                                                \
     fa##E[0] = ov_src[gi_];                                                                                          \
@@ -414,8 +414,9 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
         const bool own = sc == c;
         float gs = 0.f;  // decay between the source chunk and this chunk
         for (int x = (IS_DV ? c : sc); x < (IS_DV ? sc : c); ++x) gs += graw[x];
-        // exponent offset of this lane's position, in powers of two, with the 1/sqrt(d) of the scores folded in
-        const float un2 = (nv + (IS_DV ? -gs : gs)) * kLog2e + (IS_DV ? -1.f : 1.f) * __log2f(a.qk_scale);
+        // gate exponent of this lane's position; the 1/sqrt(d) of the scores rides in the exponent (lq)
+        const float un = nv + (IS_DV ? -gs : gs);
+        const float lq = __log2f(a.qk_scale);
 #pragma unroll
         for (int kh = 0; kh < 2; ++kh) {
           // the two halves use the ring slots the other way round (three slabs per half)
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
               for (int q = 0; q < 4; ++q) {
                 const int o = 64 * kh + ol + q;
                 // exp(u_t - w_j + G) / sqrt(d) as one power of two
-                const float e2 = __builtin_amdgcn_exp2f(IS_DV ? (xov[q] - un2) : (un2 - xov[q]));
+                const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(IS_DV ? (xov[q] - un) : (un - xov[q]), kLog2e, lq));
                 const bool keep = !own || (IS_DV ? (n <= o) : (o <= n));
                 float val = sacc[4 * g4 + q] * e2;
                 if (IS_DV) val *= rho[q];

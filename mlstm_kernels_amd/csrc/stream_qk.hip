@@ -69,7 +69,7 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
   extern __shared__ __align__(16) unsigned char smem_raw[];
   uint16_t* const Ring = (uint16_t*)smem_raw;     // [3][SLOT]
   uint16_t* const Ps = Ring + 3 * SLOT;
-  float* const ovec = (float*)(Ps + 128 * PS);    // [128] gate vector of the source chunk times log2(e): w_j (dQ) / u_t (dK)
+  float* const ovec = (float*)(Ps + 128 * PS);    // [128] gate vector of the source chunk: w_j (dQ) / u_t (dK)
   float* const orho = ovec + 128;                 // [128] dK: rho_t of the source chunk (dQ: ones)
   float* const red = orho + 128;                  // [4][128] row-dot partials of the previous item, per 64-row block
 
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
     const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
     _Pragma("unroll") for (int i_ = 0; i_ < 8; ++i_) *(u32x4*)(smem_raw + d0_ + i_ * step_) = fd##E[i_];             \
     if (__builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 128) {                                          \
-      ovec[p] = fa##E[0] * kQkLog2e;                                                                                 \
+      ovec[p] = fa##E[0];                                                                                 \
       orho[p] = __builtin_amdgcn_readfirstlane((int)((w_ >> 23) & 1)) ? 1.f / (fa##E[1] + a.eps) : 1.f;              \
     }                                                                                                                \
   }
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
     const uint32_t d0_ = w_ & 0xFFFFFu;                                                                              \
     const bool st_ = L >= 2;                                                                                         \
     if (st_ && __builtin_amdgcn_readfirstlane((int)((w_ >> 22) & 1)) && p < 128) {                                   \
-      ovec[p] = fa##E[0] * kQkLog2e;                                                                                 \
+      ovec[p] = fa##E[0];                                                                                 \
       orho[p] = __builtin_amdgcn_readfirstlane((int)((w_ >> 23) & 1)) ? 1.f / (fa##E[1] + a.eps) : 1.f;              \
     }                                                                                                                \
     fa##E[0] = ov_src[gi_];                                                                                          \
@@ -280,7 +280,8 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
     float gs = 0.f; /* decay between the two chunks */                                                               \
     for (int x = (dk ? c : (sc_)); x < (dk ? (sc_) : c); ++x) gs += graw[x];                                         \
     const float sgn = dk ? -1.f : 1.f;                                                                               \
-    const float un2 = (nv + sgn * gs) * kQkLog2e + sgn * __log2f(a.qk_scale);                                        \
+    const float un = nv + sgn * gs;                                                                                  \
+    const float lq = __log2f(a.qk_scale);                                                                            \
     const int le = opaque(lane);                                                                                     \
     const int r = le & 31, h = le >> 5;                                                                              \
     const int n = 32 * nbk + r;                                                                                      \
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(768) void stream_qk_kernel(ParQkArgs a, int n_items
       const float rov[4] = {ro.x, ro.y, ro.z, ro.w};                                                                 \
       float pv[4];                                                                                                   \
       _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                                                \
-        const float e2 = __builtin_amdgcn_exp2f(sgn * (un2 - xov[q]));                                               \
+        const float e2 = __builtin_amdgcn_exp2f(__builtin_fmaf(sgn * (un - xov[q]), kQkLog2e, lq));                  \
         const bool keep = !(OWN_) || (dk ? (n <= o0 + q) : (o0 + q <= n));                                           \
         const float val = sacc[kk][4 * g4 + q] * e2 * (nrho * rov[q]);                                               \
         pv[q] = keep ? val : 0.f;                                                                                    \

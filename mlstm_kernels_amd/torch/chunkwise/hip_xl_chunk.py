@@ -47,7 +47,7 @@ def _warn_rounding_once(dtype: torch.dtype) -> None:
         )
 
 
-def _state_stride(tuning_kwargs: dict, who: str) -> int:
+def _state_stride(tuning_kwargs: dict, who: str, chunk_size: int = 128) -> int:
     """chunk_size_inter / chunk_size_intra of the reference (kernel_param_heuristics.py:118-121) -> state stride.
 
     The reference scans in chunks of chunk_size_inter and keeps a state every chunk_size_intra positions.  The HIP
@@ -63,6 +63,12 @@ def _state_stride(tuning_kwargs: dict, who: str) -> int:
     if inter is not None and inter not in (16, 32, 64, _INTERNAL_CHUNK):
         raise ValueError(f"chunk_size_inter must be 16, 32, 64 or {_INTERNAL_CHUNK} (or None), got {inter}")
     if intra is None:
+        # the reference takes chunk_size as chunk_size_intra when the latter is not given
+        # (kernel_param_heuristics.py:96-121): a caller who asks for chunks of 256 positions or more gets a kept state
+        # every chunk_size positions (at most every 1024); the reference's default of 128 leaves the choice to the
+        # library (a state every 256 positions, the measured optimum on MI355X: same results, half the workspace)
+        if isinstance(chunk_size, int) and chunk_size >= 2 * _INTERNAL_CHUNK and chunk_size % _INTERNAL_CHUNK == 0:
+            return min(chunk_size // _INTERNAL_CHUNK, 8)
         return 0
     if inter is not None and (intra < inter or intra % inter != 0):
         raise ValueError(f"chunk_size_intra ({intra}) must be a multiple of chunk_size_inter ({inter})")
@@ -297,18 +303,25 @@ def mlstm_chunkwise__hip_xl_chunk(
 ):
     """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
     ``(H, (C_last fp32 (B,NH,DHQK,DHHV), n_last fp32 (B,NH,DHQK), m_last fp32 (B,NH,1)))``.
-    The matrix kernels multiply in the dtype of q -- bfloat16 or float16 -- with fp32 accumulation; float32 inputs
-    are rounded to bfloat16, with a one-time warning.
+    Two defaults differ from the reference behind the same signature (the results do not): ``recompute_states_in_bw``
+    defaults to False here (True in mlstm_kernels/torch/chunkwise/triton_xl_chunk/fwbw.py:266; keeping the states
+    holds 0.56 GB more between the passes at the benchmark shape and is 0.35 ms faster), and
+    ``autocast_kernel_dtype=torch.float32`` -- the reference's default, for which it instantiates a float32 kernel
+    (fwbw.py:222-241) -- means bfloat16 OPERANDS here: the matrix kernels multiply in the dtype of q, bfloat16 or
+    float16, with fp32 accumulation, gates, normalisers and states; float32 inputs are rounded to bfloat16 with a
+    one-time warning (about 1e-2 relative error in H against the float32 recurrence on the unrounded inputs).
+    ``chunk_size`` is validated like the reference does; 256 or more also sets the distance between kept states
+    (as the reference's chunk_size_intra default does), 128 leaves it to the library.
     ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
-    tail themselves, so every S >= 1 is one call.  ``kernel_path`` ("auto", "split", "fused"; not in the reference)
-    selects the kernels of the value-column side.  ``chunk_size_intra`` (reference keyword) sets the distance between
+    tail themselves, so every S >= 1 is one call.  ``kernel_path`` ("auto", "split", "stream", "fused"; not in the
+    reference) selects the kernels of the chunk-parallel passes.  ``chunk_size_intra`` (reference keyword) sets the distance between
     kept chunk states; ``recompute_states_in_bw=True`` (reference keyword) keeps none of them between forward and
     backward.  ``head_norm`` ("none", "layer", "rms"; not in the reference's operator) fuses the multi-head
     norm that follows the cell in the xLSTM block -- the reference's ``apply_normalize(norm_specifier, x, eps)``,
     mlstm_kernels/utils/analysis/transfer_behavior/_norm_layers.py:11-64, over the DHHV columns of every row, without
     scale parameters -- into the output kernel: the returned ``H`` is then the normalised one and the un-normalised
     output never goes to memory (DHHV = 64, 128, 256 or 512)."""
-    stride = _state_stride(tuning_kwargs, "mlstm_chunkwise__hip_xl_chunk")
+    stride = _state_stride(tuning_kwargs, "mlstm_chunkwise__hip_xl_chunk", chunk_size)
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
     fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride, head_norm, head_norm_eps,
@@ -341,7 +354,7 @@ def mlstm_siging_chunkwise__hip_xl_chunk(
 ):
     """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``.
     ``any_sequence_length``, ``kernel_path``, ``chunk_size_intra`` and ``head_norm`` as for the exp gate."""
-    stride = _state_stride(tuning_kwargs, "mlstm_siging_chunkwise__hip_xl_chunk")
+    stride = _state_stride(tuning_kwargs, "mlstm_siging_chunkwise__hip_xl_chunk", chunk_size)
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
     fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride, head_norm, head_norm_eps,

@@ -89,7 +89,8 @@ def mlstm_recurrent_step__hip(
     dtype_state: torch.dtype = torch.float32,
     **kwargs,
 ):
-    """Single mLSTM step: returns ``h (B,NH,DHHV)`` in q's dtype and ``(C', n', m')`` in float32."""
+    """Single mLSTM step: returns ``h (B,NH,DHHV)`` in q's dtype and ``(C', n', m')`` in ``dtype_state`` (float32 unless
+    asked otherwise; the arithmetic is float32 either way and h is formed from the unrounded new state)."""
     return mlstm_recurrent_step__hip_fw(
         matC_old=c, vecN_old=n, scaM_old=m, vecQ=q, vecK=k, vecV=v, scaI=i, scaF=f,
         eps=eps, dtype_state=dtype_state, **kwargs,
@@ -113,7 +114,16 @@ def mlstm_recurrent_sequence__hip(
     """All S tokens in one launch of the multi-token kernel: the state stays on chip between tokens and moves
     through HBM once each way for the whole sequence (a loop of single steps moves it once each way per token).
     Used for multi-token decode and for the short remainder of a prefill.  Same arguments and return structure
-    as mlstm_recurrent_sequence__triton_step_fused_fw (mlstm_kernels/torch/recurrent/native_sequence.py:86-122)."""
+    as mlstm_recurrent_sequence__triton_step_fused_fw (mlstm_kernels/torch/recurrent/native_sequence.py:86-122), with
+    two differences that are stated here rather than hidden: ``return_all_states=True`` (the state after every token,
+    native_sequence.py:20,64-83) is not implemented and raises; with a 16-bit ``dtype_state`` the state is rounded
+    once per call -- it stays float32 in registers between the tokens -- where the reference's token loop rounds it
+    after every step (the results of that mode are therefore closer to the float32 recurrence, not bit-equal)."""
+    if kwargs.pop("return_all_states", False):
+        raise NotImplementedError("mlstm_recurrent_sequence__hip does not return the state after every token "
+                                  "(return_all_states=True); loop over mlstm_recurrent_step__hip for that")
+    if kwargs:
+        raise TypeError(f"mlstm_recurrent_sequence__hip() got unexpected keyword arguments {sorted(kwargs)}")
     B, NH, S, DHQK = q.shape
     DHHV = v.shape[-1]
     assert k.shape == q.shape, "q and k must have the same shape"

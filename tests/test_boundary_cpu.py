@@ -267,3 +267,47 @@ def test_reference_kernel_names_are_opt_in_aliases():
         T._extra_kernels.clear(), T._extra_kernels.update(saved[0])
         T._extra_step.clear(), T._extra_step.update(saved[1])
         T._extra_sequence.clear(), T._extra_sequence.update(saved[2])
+
+
+def test_noalloc_scratch_size_matches_the_header():
+    """_lib.NOALLOC_SCRATCH_BYTES mirrors MLSTM_NOALLOC_SCRATCH_BYTES of include/mlstm_hip.h: parsed here, not retyped."""
+    import os
+    import re
+
+    from mlstm_kernels_amd import _lib
+
+    header = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "mlstm_hip.h")).read()
+    m = re.search(r"#define\s+MLSTM_NOALLOC_SCRATCH_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)", header)
+    assert m, "MLSTM_NOALLOC_SCRATCH_BYTES not found in the header"
+    assert int(m.group(1)) << int(m.group(2)) == _lib.NOALLOC_SCRATCH_BYTES
+    for name, code in (("MLSTM_PATH_AUTO", _lib.PATH_AUTO), ("MLSTM_PATH_SPLIT", _lib.PATH_SPLIT),
+                       ("MLSTM_PATH_FUSED", _lib.PATH_FUSED), ("MLSTM_PATH_STREAM", _lib.PATH_STREAM)):
+        m = re.search(r"#define\s+" + name + r"\s+(\d+)", header)
+        assert m and int(m.group(1)) == code, name
+
+
+def test_chunk_size_sets_the_state_stride_like_the_reference_default():
+    """chunk_size_intra defaults to the target chunk size in the reference (kernel_param_heuristics.py:96-121): 256 or
+    more therefore names the distance between kept states here too; 128 leaves it to the library."""
+    from mlstm_kernels_amd.torch.chunkwise.hip_xl_chunk import _state_stride
+
+    assert _state_stride({}, "op", 128) == 0
+    assert _state_stride({}, "op", 64) == 0
+    assert _state_stride({}, "op", 256) == 2
+    assert _state_stride({}, "op", 512) == 4
+    assert _state_stride({}, "op", 2048) == 8
+    assert _state_stride({"chunk_size_intra": 128}, "op", 512) == 1   # an explicit value wins
+
+
+def test_recurrent_sequence_rejects_what_it_does_not_implement():
+    import pytest
+    import torch
+
+    from mlstm_kernels_amd.torch.recurrent import mlstm_recurrent_sequence__hip
+
+    t = torch.zeros(1, 1, 2, 64)
+    g = torch.zeros(1, 1, 2)
+    with pytest.raises(NotImplementedError, match="return_all_states"):
+        mlstm_recurrent_sequence__hip(t, t, t, g, g, return_all_states=True)
+    with pytest.raises(TypeError, match="unexpected keyword"):
+        mlstm_recurrent_sequence__hip(t, t, t, g, g, no_such_option=1)

@@ -6,7 +6,8 @@ Stated tolerances (bf16 inputs, fp32 states):
     (gated scores, chunk states) to the matrix cores: one operand of every product carries a relative rounding error
     of up to 2^-8 (8-bit significand).  On rows whose normaliser nearly cancels the products are large against their
     sum and that rounding exceeds the bound on a few elements in 10^4.  The tests therefore require
-      - the bound on >= 99.9 % of the elements, max|x - ref| <= 1e-2 max|ref|, ||x - ref|| <= 5e-3 ||ref||, and
+      - the bound on all but 3 in 10^4 elements of H and dV and 1 in 10^3 of dQ and dK (twice the measured rates), the
+        worst element within 8 x the bound (dK 16 x), max|x - ref| <= 1e-2 max|ref|, ||x - ref|| <= 5e-3 ||ref||, and
       - on EVERY element |x - ref| <= 2e-2 + 2e-2 |ref| + 1.25 * 2^-8 * A, where A is the sum of the magnitudes of all
         products entering that element (computed by the oracle in the same chunk decomposition): the first-order
         worst case of the operand roundings.  The count of offenders and the worst one are printed per tensor.
@@ -96,15 +97,28 @@ _U_BF16 = 2.0 ** -8   # unit roundoff of an 8-bit significand
 _U_F16 = 2.0 ** -11   # ... of an 11-bit significand
 
 
-def check_matrix(x, ref, name, frac=1e-3, scale_tol=1e-2, norm_tol=5e-3, worst_tol=16.0, abs_sum=None, unit=_U_BF16):
+# Allowance outside the plain 2e-2/2e-2 bound per tensor: at most twice the rate measured at the full benchmark shapes
+# (H, dV: 0.7-1.6 per 10^4 elements; dQ, dK: 2.3-5.8 per 10^4), and the worst element within 8 x the bound (dK: 16 x;
+# one dK element with nearly cancelling terms measures 13.0 x).  The COUNT of offenders is held to that rate plus three
+# standard deviations of a Poisson count plus two elements, so that tensors of a few thousand elements are not judged
+# on two or three elements.
+_FRAC = {"H": 3e-4, "dV": 3e-4, "dQ": 1e-3, "dK": 1e-3}
+_WORST = {"H": 8.0, "dV": 8.0, "dQ": 8.0, "dK": 16.0}
+
+
+def check_matrix(x, ref, name, frac=None, scale_tol=1e-2, norm_tol=5e-3, worst_tol=None, abs_sum=None, unit=_U_BF16):
     """`abs_sum` (same shape as ref): magnitude sum of the products entering each element; when given, every element
     must lie within the 2e-2/2e-2 bound widened by the worst case of one operand rounding (unit roundoff `unit`) per
     product."""
+    key = name.split()[0].split("(")[0]
+    frac = _FRAC.get(key, 1e-3) if frac is None else frac
+    worst_tol = _WORST.get(key, 16.0) if worst_tol is None else worst_tol
     bad, worst = report_offenders(x, ref, name)
     e1, e2 = rel_to_scale(x, ref), rel_norm(x, ref)
-    assert bad <= frac and worst <= worst_tol and e1 <= scale_tol and e2 <= norm_tol, (
-        f"{name}: {bad:.2e} of elements outside 2e-2/2e-2 (worst {worst:.2f} x the bound), max err / scale {e1:.2e}, "
-        f"norm err {e2:.2e}")
+    n_allowed = frac * ref.numel() + 3.0 * (frac * ref.numel()) ** 0.5 + 2.0
+    assert bad * ref.numel() <= n_allowed and worst <= worst_tol and e1 <= scale_tol and e2 <= norm_tol, (
+        f"{name}: {bad:.2e} of elements outside 2e-2/2e-2 (allowed {frac:.1e}; worst {worst:.2f} x the bound, allowed "
+        f"{worst_tol:g}), max err / scale {e1:.2e}, norm err {e2:.2e}")
     if abs_sum is not None:
         x64, r64 = x.detach().double().cpu(), ref.detach().double().cpu()
         slack = (x64 - r64).abs() - (2e-2 + 2e-2 * r64.abs() + 1.25 * unit * abs_sum.double().cpu())
@@ -443,6 +457,46 @@ def test_last_state_accuracy_across_decay_regimes(f_offset):
     assert_state_close(n, ref["n_last"], 1e-4, "n_last")
 
 
+def test_last_state_accuracy_sig_gate_with_closed_late_inputs():
+    """Sigmoid input gate, input gate shut over the last two chunks: the early chunks then dominate C_last although
+    their decay weight is small, and without a stabiliser the decay factors alone do not show that -- every chunk of a
+    sigmoid-gate scan therefore carries the remainder of the value operand.  C_last and n_last to 1e-3."""
+    if _VARIANT["kernel_path"] == "fused":
+        pytest.skip("the remainder split is the split and stream paths' scan")
+    _, sig_op, *_ = _ops()
+    B, NH, S, DQK, DHV = 1, 2, 1024, 128, 256
+    q, k, v, i, f = make_qkvif(B, NH, S, DQK, DHV, seed=77)
+    f = f - 2.0                       # forget gates around 1: sigmoid(1) ~ 0.73, weight of early chunks ~ 1e-35 .. 1e-17
+    i = i.clone()
+    i[:, :, -256:] = -14.0            # closed input gate over the last two chunks
+    H, (C, n) = sig_op(*(t.to(DEV) for t in (q, k, v, i, f)), return_last_states=True, chunk_size=128)
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=128, siging=True)
+    assert_state_close(C, ref["C_last"], 1e-3, "C_last")
+    assert_state_close(n, ref["n_last"], 1e-3, "n_last")
+
+
+def test_float32_inputs_run_with_bfloat16_operands():
+    """autocast_kernel_dtype=torch.float32 (the reference's default, for which it instantiates a float32 kernel:
+    mlstm_kernels/torch/chunkwise/triton_xl_chunk/fwbw.py:222-241,267) means bfloat16 OPERANDS here.  Inputs with full
+    float32 mantissas against the fp64 oracle on the UNROUNDED values: the error is that of rounding q, k and v to
+    bfloat16 on top of the bfloat16 path's own roundings (measured: norm error 1.3e-2, 1.2 % of the elements outside
+    2e-2/2e-2, worst 8.4 x the bound), not float32's (which would be ~1e-6); pinned from both sides so that a change of
+    the operand format shows up here."""
+    exp_op, *_ = _ops()
+    B, NH, S, DQK, DHV = 1, 2, 512, 256, 512
+    g = torch.Generator().manual_seed(123)
+    q, k, v = (torch.randn(B, NH, S, d, generator=g) for d in (DQK, DQK, DHV))   # float32, not bf16-representable
+    i, f = torch.randn(B, NH, S, generator=g), 3 + torch.randn(B, NH, S, generator=g)
+    assert (q.bfloat16().float() != q).any()
+    H = exp_op(*(t.to(DEV) for t in (q, k, v, i, f)), chunk_size=128, autocast_kernel_dtype=torch.float32)
+    assert H.dtype == torch.float32
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=128)
+    check_matrix(H, ref["H"], "H", frac=3e-2, worst_tol=16.0, scale_tol=1e-1, norm_tol=2e-2)
+    e = rel_norm(H, ref["H"])
+    print(f"    float32 inputs: norm error {e:.2e}")
+    assert 5e-3 <= e <= 2e-2, f"norm error {e:.2e}: not the bfloat16 operand path's"
+
+
 def test_unsupported_head_dim_fails_loudly():
     exp_op, *_ = _ops()
     for dqk in (960, 1024):
@@ -666,6 +720,47 @@ def test_chunkwise_takes_16_bit_gates(dtype, siging):
         assert rel_to_scale(leaf.grad, r) <= 5e-2, name
 
 
+@pytest.mark.parametrize("stride,recompute,init", [(3, False, False), (8, True, True)])
+def test_long_sequence_with_rarely_kept_states(stride, recompute, init, kernel_variant):
+    """State strides 3 and 8 on a sequence of 32 chunks (11 and 4 kept states per pass; the scan's decay table is
+    refilled on the way): forward and backward against the oracle on one (batch, head) pair, once with the reference's
+    saved-state policy (recompute_states_in_bw=True, mlstm_kernels/torch/chunkwise/triton_xl_chunk/bw.py:75-95) and a
+    non-zero initial state.  The other tests reach these strides only through the random sweep at S <= 777."""
+    if kernel_variant not in ("split-1", "stream-1"):
+        pytest.skip("runs once per kernel path (the stride is this test's own parameter)")
+    from mlstm_kernels_amd.torch.chunkwise import mlstm_chunkwise__hip_xl_chunk as op
+
+    B, NH, S, DQK, DHV = 1, 2, 4096, 256, 512
+    gpu_gen = torch.Generator(device=DEV).manual_seed(100 + stride)
+    rn = lambda *s: torch.randn(*s, device=DEV, generator=gpu_gen)
+    q, k, v, dH = (rn(B, NH, S, d).bfloat16() for d in (DQK, DQK, DHV, DHV))
+    i, f = rn(B, NH, S), 3 + rn(B, NH, S)
+    c0 = n0 = m0 = None
+    if init:
+        c0, n0, m0 = 0.1 * rn(B, NH, DQK, DHV), 0.1 * rn(B, NH, DQK), torch.zeros(B, NH, 1, device=DEV)
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, i, f)]
+    c0l = None if c0 is None else c0.clone().requires_grad_(True)
+    H = op(*leaves, c_initial=c0l, n_initial=n0, m_initial=m0, chunk_size=128, chunk_size_intra=128 * stride,
+           kernel_path=kernel_variant.split("-")[0], recompute_states_in_bw=recompute)
+    H.backward(dH)
+    b, h = 0, 1
+    sl = lambda t: None if t is None else d64(t[b:b + 1, h:h + 1])
+    L = 128 * stride
+    bounded = S % L == 0   # the oracle's magnitude sums describe the kernels' grouping only then
+    Lo = L if bounded else 128
+    fw = O.chunkwise_fw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(c0), sl(n0), sl(m0), chunk_size=Lo, return_bounds=True)
+    bw = O.chunkwise_bw(sl(q), sl(k), sl(v), sl(i), sl(f), sl(dH), sl(c0), sl(n0), sl(m0), None, chunk_size=Lo,
+                        return_bounds=True)
+    check_matrix(H[b:b + 1, h:h + 1], fw["H"], "H", abs_sum=fw["H_abs"] if bounded else None)
+    for name, leaf, r in zip(["dQ", "dK", "dV"], leaves[:3], bw[:3]):
+        check_matrix(leaf.grad[b:b + 1, h:h + 1], r, name, abs_sum=bw[6][name + "_abs"] if bounded else None)
+    for name, leaf, r in zip(["dI", "dF"], leaves[3:], bw[3:5]):
+        e = rel_to_scale(leaf.grad[b:b + 1, h:h + 1], r)
+        assert e <= 5e-2, f"{name}: max err / scale {e:.2e}"
+    if c0l is not None:
+        assert rel_norm(c0l.grad[b:b + 1, h:h + 1], bw[5]) <= 5e-3, "dC0"
+
+
 @pytest.mark.parametrize("kw", [
     dict(B=2, NH=2, S=1024, DQK=256, DHV=512, seed=50),
     dict(B=1, NH=2, S=640, DQK=128, DHV=256, seed=51, init=True, last=True),
@@ -698,6 +793,10 @@ def test_recompute_states_in_bw_matches_kept_states(kw, kernel_variant):
     def run(recompute):
         leaves = [t.to(DEV).requires_grad_(True) for t in (q, k, v, i, f)]
         c0l = c0.clone().requires_grad_(True) if init else None
+        # (tensors of earlier tests that the collector has not freed yet must not be freed inside the measured span)
+        import gc
+
+        gc.collect()
         torch.cuda.synchronize()
         base = torch.cuda.memory_allocated()
         out = op(*leaves, c_initial=c0l, n_initial=n0, m_initial=m0, return_last_states=last, chunk_size=128,

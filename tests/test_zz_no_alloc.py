@@ -60,6 +60,47 @@ def test_noalloc_forward_matches_the_workspace_entry_point_on_two_calls_in_a_row
         assert not torch.isnan(got[0].float()).any()
 
 
+def test_noalloc_forward_in_a_hip_graph_after_one_eager_call():
+    """The entry point is meant for callers under HIP graph capture.  Its first call on a device looks the scratch
+    address up and sets kernel attributes (host-side work that does not belong into a capture), so ONE eager call per
+    device and shape comes first; after it the call is captured and replayed, with eager work between the replays:
+    every replay reproduces the eager result bit for bit."""
+    from mlstm_kernels_amd import _lib
+    from mlstm_kernels_amd.torch.utils import current_stream_ptr, ptr
+
+    lib = _lib.get_lib()
+    dev = torch.device("cuda")
+    B, NH, S, DHQK, DHHV = 1, 4, 1024, 256, 512
+    g = torch.Generator(device=dev).manual_seed(7)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    q, k, v = rn(B, NH, S, DHQK).bfloat16(), rn(B, NH, S, DHQK).bfloat16(), rn(B, NH, S, DHHV).bfloat16()
+    i, f = rn(B, NH, S), 3 + rn(B, NH, S)
+    H = torch.empty(B, NH, S, DHHV, dtype=torch.bfloat16, device=dev)
+    c_last, n_last, m_last = torch.empty(B, NH, DHQK, DHHV, device=dev), torch.empty(B, NH, DHQK, device=dev), torch.empty(B, NH, device=dev)
+
+    def call():
+        rc = lib.mlstm_hip_chunkwise_fw_noalloc(ptr(q), ptr(k), ptr(v), ptr(i), ptr(f), None, None, None, ptr(H), None, None,
+                                                ptr(c_last), ptr(n_last), ptr(m_last), B, NH, S, DHQK, DHHV, 1e-6, _lib.BF16,
+                                                _lib.F32, _lib.GATE_EXP, 1, current_stream_ptr(dev))
+        _lib.check(rc, "mlstm_hip_chunkwise_fw_noalloc")
+
+    call()  # the eager warm-up call
+    torch.cuda.synchronize()
+    H_ref, c_ref = H.clone(), c_last.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        H.zero_()
+        c_last.zero_()
+        q2 = (q.float() * 0.5).bfloat16()   # eager work of the program's own between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(H, H_ref) and torch.equal(c_last, c_ref), f"replay {rep} differs from the eager call"
+    del q2
+
+
 def test_noalloc_forward_rejects_shapes_beyond_the_static_scratch():
     from mlstm_kernels_amd import _lib
     from mlstm_kernels_amd.torch.utils import current_stream_ptr, ptr
