@@ -20,6 +20,13 @@ Objects on the JSON line besides the contract's keys:
   peak_memory_gb -- peak device memory of one forward+backward pass (inputs, outputs, gradients, workspaces; without
                    the benchmark's own flush buffer); the reference's benchmark reports 9.0-9.9 GB for this workload.
   roofline_hbm  -- the same kernel against the HBM peak (algorithmic bytes per launch).
+  roofline_step -- the whole forward+backward step against the HBM peak: algorithmic bytes if every operand moved once
+                   and no chunk state travelled (4.31 GB), algorithmic bytes of this kernel decomposition (with the
+                   kept chunk states), bytes measured by rocprofv3 (FETCH_SIZE + WRITE_SIZE summed over the five matrix
+                   kernels, from profiles/), achieved GB/s = measured bytes / ms_per_step and its fraction of the
+                   peak, and executed over algorithmic matrix flops (SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512, from
+                   profiles/).  `profile_kernel_ms` are the kernel durations of the profiled run: the counters describe
+                   this run only where they agree with `kernels` (`profile_matches_run`).
   kernels       -- average duration, algorithmic TFLOP/s and GB/s of every kernel of the step.
   decode_step   -- fused decode step at B=256 after a chunkwise prefill of 2048 positions: ms per step, algorithmic
                    GB/s, its own HBM roofline; B=64 and B=16 (whose state fits the memory-side cache: "bound": "mall");
@@ -73,6 +80,11 @@ STEP_BYTES_PER_BH = 2 * DHQK * DHHV * 4 + 2 * DHQK * 4 + 2 * 4 + (2 * DHQK + DHH
 DECODE_B, DECODE_PREFILL, DECODE_STEPS, DECODE_WARMUP = 256, 2048, 128, 10
 MALL_BYTES = 256 << 20
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "tfla_fwbw_B4_S16384__pmc_hbm_traffic.md")
+SQ_PROFILE = os.path.join(ROOT, "profiles", "tfla_fwbw_B4_S16384__pmc_sq_counters.md")
+MATRIX_KERNELS = ("scan_fw", "par_h", "scan_bw", "par_dv", "par_dqdk")
+# minimal HBM bytes per token and head: forward q, k, v in, H out, i, f (3076); backward q, k, v, dH, i, f in, dQ, dK,
+# dV, dI, dF out (5136)
+IO_ONCE_BYTES_PER_TOKEN_HEAD = 3076 + 5136
 
 
 def algorithmic_bytes(stride: int) -> dict:
@@ -98,6 +110,24 @@ def measured_traffic() -> dict:
     for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
         out[m.group(1)] = float(m.group(4)) * 1e6
     return out
+
+
+def measured_mfma_flops() -> dict:
+    """{kernel: executed matrix flops per launch} from the SQ counter summary under profiles/ (column MFMA MOPS, units
+    of 512 flop), and {kernel: ms} the durations of that profiled run (row `profiled run, ms per launch`)."""
+    flops, ms = {}, {}
+    try:
+        text = open(SQ_PROFILE).read()
+    except OSError:
+        return flops, ms
+    for line in text.splitlines():
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 9 and cells[0] in MATRIX_KERNELS and cells[7].isdigit():
+            flops[cells[0]] = int(cells[7]) * 512.0
+    m = re.search(r"profiled run, ms per launch:\s*(\{.*\})", text)
+    if m:
+        ms = json.loads(m.group(1))
+    return flops, ms
 
 
 def cpu_model() -> str:
@@ -291,6 +321,30 @@ def main():
             entry["hbm_bytes_measured"] = traffic[name]
             entry["measured_gbs"] = round(traffic[name] / (entry["avg_ms"] * 1e-3) / 1e9, 1)   # rocprofv3 bytes / this run's time
 
+    # ---- the whole step against the HBM roofline
+    mfma_flops, prof_ms = measured_mfma_flops()
+    have_all = all(k in traffic for k in MATRIX_KERNELS)
+    step_bytes_measured = sum(traffic[k] for k in MATRIX_KERNELS) if have_all else None
+    io_once = IO_ONCE_BYTES_PER_TOKEN_HEAD * TOKEN_HEADS
+    roofline_step = {
+        "bound": "hbm", "algorithmic_bytes_io_once": io_once,
+        "algorithmic_bytes_this_decomposition": sum(alg_bytes.values()),
+        "measured_bytes": step_bytes_measured, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+        "achieved": None if step_bytes_measured is None else round(step_bytes_measured / (ms_per_step * 1e-3) / 1e9, 1),
+        "frac": None if step_bytes_measured is None else round(step_bytes_measured / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+        "achieved_io_once": round(io_once / (ms_per_step * 1e-3) / 1e9, 1),
+        "frac_io_once": round(io_once / (ms_per_step * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+        "mfma_flops_executed": sum(mfma_flops.values()) if all(k in mfma_flops for k in MATRIX_KERNELS) else None,
+        "mfma_flops_algorithmic": (FLOPS_FW + FLOPS_BW) * TOKEN_HEADS,
+        "profile_kernel_ms": prof_ms or None,
+        "source": "profiles/tfla_fwbw_B4_S16384__pmc_hbm_traffic.md, profiles/tfla_fwbw_B4_S16384__pmc_sq_counters.md",
+    }
+    if roofline_step["mfma_flops_executed"]:
+        roofline_step["executed_over_algorithmic_flops"] = round(roofline_step["mfma_flops_executed"] / roofline_step["mfma_flops_algorithmic"], 3)
+    if prof_ms:
+        roofline_step["profile_matches_run"] = all(
+            k in kernels and abs(kernels[k]["avg_ms"] - prof_ms[k]) <= 0.2 * prof_ms[k] for k in MATRIX_KERNELS if k in prof_ms)
+
     extra = {}
     if not args.no_extra:
         n_extra = max(5, args.steps // 2)
@@ -441,7 +495,7 @@ def main():
                    "mean_ms": round(head["mean_ms"], 4), "min_ms": round(head["min_ms"], 4),
                    "wall_ms_per_step_incl_flush": round(head["wall_ms_incl_flush"], 4)},
         "peak_memory_gb": head["peak_memory_gb"], "peak_memory_beyond_inputs_gb": head["peak_memory_beyond_inputs_gb"],
-        "roofline": roofline, "roofline_hbm": roofline_hbm, "kernels": kernels, "decode_step": decode, "extra": extra,
+        "roofline": roofline, "roofline_hbm": roofline_hbm, "roofline_step": roofline_step, "kernels": kernels, "decode_step": decode, "extra": extra,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
