@@ -13,7 +13,10 @@
  *   - dtype codes: MLSTM_F32 = 0, MLSTM_BF16 = 1, MLSTM_F16 = 2.  The chunkwise entry points take q/k/v (and dH) in
  *     bf16 or fp16 and multiply in that format on the matrix cores with fp32 accumulation (the kept chunk states are
  *     rounded to the same format; fp16 has three more mantissa bits and overflows above 65504); gates in fp32, bf16 or
- *     fp16.  The decode entry points take q/k/v, gates and states in fp32, bf16 or fp16 each (fp32 arithmetic).
+ *     fp16.  MLSTM_F32 is rejected for the q/k/v of a chunkwise call: there is no fp32 matrix path.  (The Python host
+ *     code converts float32 tensors to bf16 before the call, so a float32 call there computes with bf16 operands --
+ *     about 1e-2 relative error of the outputs in norm -- and not in the fp32 arithmetic of the reference's float32
+ *     configuration.)  The decode entry points take q/k/v, gates and states in fp32, bf16 or fp16 each (fp32 arithmetic).
  *   - gate codes: MLSTM_GATE_EXP = 0 (mLSTMexp), MLSTM_GATE_SIG = 1 (mLSTMsig, sigmoid input gate).
  *   - Supported shapes: DHQK % 64 == 0 (at most 896), DHHV % 64 == 0, any S >= 1 (the kernels mask the ragged tail).
  *
@@ -199,6 +202,9 @@ int mlstm_hip_head_norm_bw(const void* dY, const void* Y, const float* rstd, voi
  * ends) instead of a caller-provided buffer.  The call allocates and frees nothing.  Shapes whose workspace
  * (mlstm_hip_chunkwise_fw_workspace_bytes(B, NH, S, DHQK, DHHV, 0, MLSTM_PATH_AUTO, 0)) exceeds the static scratch are
  * rejected.  All calls on one GPU share that GPU's scratch: calls that overlap in time on one GPU race.
+ * Under HIP graph capture: make one eager call of the same shape on the device before the capture begins.  The first
+ * call on a device looks up the scratch address (hipGetSymbolAddress), the number of CUs and the kernels' LDS limits
+ * (hipFuncSetAttribute), none of which a capturing stream records; later calls only launch kernels.
  */
 #define MLSTM_NOALLOC_SCRATCH_BYTES (64u << 20)
 int mlstm_hip_chunkwise_fw_noalloc(const void* q, const void* k, const void* v, const void* i, const void* f,

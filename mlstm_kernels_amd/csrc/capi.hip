@@ -6,6 +6,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -23,7 +24,7 @@ struct TimedLaunch {
   hipEvent_t start, stop;
 };
 std::mutex g_prof_mutex;
-bool g_prof_on = false;
+std::atomic<bool> g_prof_on{false};   // read by every launch, written by mlstm_profile_enable from any thread
 std::vector<TimedLaunch> g_prof_launches;
 
 struct ProfileScope {
@@ -32,7 +33,7 @@ struct ProfileScope {
   hipEvent_t start = nullptr, stop = nullptr;
   bool active = false;
   ProfileScope(const char* n, hipStream_t s) : name(n), stream(s) {
-    if (!g_prof_on) return;
+    if (!g_prof_on.load(std::memory_order_relaxed)) return;
     if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) return;
     active = true;
     (void)hipEventRecord(start, stream);
@@ -60,8 +61,8 @@ int check_launch(const char* what) {
 //   split : state scan, then a chunk-parallel kernel reading the materialised chunk states
 //   fused : one sequential kernel per pass that keeps the state slice in registers
 // The fused kernels move far fewer bytes (no chunk state is written or re-read by them) but run one four-wave
-// workgroup per (batch, head, 64 value columns) and per CU, which leaves them latency-bound: measured on MI355X at
-// B*S = 65536, NH = 8, 256/512 the fused forward takes 1.56 ms against 1.08 ms split.  They are opt-in only.
+// workgroup per (batch, head, 64 value columns) and per CU, which leaves them latency-bound: on MI355X at
+// B*S = 65536, NH = 8, 256/512 the fused forward is about twice as slow as scan + streaming kernel.  Opt-in only.
 bool use_fused(int path, int DHQK, int DHHV) { return path == MLSTM_PATH_FUSED && mlstm::fused_hv_supported(DHQK, DHHV); }
 // Chunk states are kept every `stride` chunks of 128 positions (0 = the default for the shape).  Fewer kept states
 // mean less HBM traffic (a state is DHQK x DHHV bf16 per chunk and head, written once and read by three kernels)
@@ -116,7 +117,7 @@ int mlstm_hip_abi_version(void) { return 6; }
 
 int mlstm_hip_profile_enable(int on) {
   std::lock_guard<std::mutex> lock(g_prof_mutex);
-  g_prof_on = on != 0;
+  g_prof_on.store(on != 0, std::memory_order_relaxed);
   return 0;
 }
 

@@ -36,8 +36,8 @@
 // Status: correct on every tested shape, but latency-bound.  With one four-wave workgroup per CU (the LDS footprint
 // allows no second one) each SIMD runs a single instruction stream, so LDS latency, vector work and matrix work
 // add up instead of overlapping: 26k cycles per chunk against 5k of matrix-pipe time.  Measured at B=4, S=16384,
-// NH=8, 256/512 on MI355X: forward 1.56 ms (scan + chunk-parallel kernel: 1.48 ms), dV 1.28 ms (1.34 ms), at a
-// third of the HBM traffic.  The host therefore selects these kernels only on request.
+// NH=8, 256/512 on MI355X: forward 1.56 ms, dV 1.28 ms, at a third of the HBM traffic of the split form, whose scan
+// plus streaming kernel take about half that time.  The host therefore selects these kernels only on request.
 #include "common.h"
 #include "kernels.h"
 

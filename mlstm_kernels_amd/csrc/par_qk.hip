@@ -26,12 +26,6 @@
 // A workgroup owns MT head-dim rows x 64 positions (half a chunk); two slabs are in flight from global memory into
 // registers while a third is being multiplied, and the footprint (54 KB of LDS) lets two workgroups share a CU so
 // that one computes while the other waits for memory.  dQ and dK run as ONE launch (par_qk_pair_kernel).
-//
-// Measured on MI355X at B=4, S=16384, 256/512 and not kept: eight waves of 32 head-dim rows per workgroup (four
-// waves per SIMD; 0.99 ms against 0.97 ms for the pair launch); dV's workgroups in the same launch as well (1.56 ms
-// against 1.52 ms for dV followed by the pair launch: they stream the shared operands in another order); the Xo score
-// operands fetched straight from global memory in fragment layout instead of through LDS (1.03 against 0.98 ms: 32-byte
-// row pieces per lane pair are a poor access pattern, the LDS detour is cheaper).
 #include "common.h"
 #include "kernels.h"
 

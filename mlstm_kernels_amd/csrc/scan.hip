@@ -33,28 +33,10 @@ constexpr int kGBlock = 256;  // chunks per refill of the decay-factor table in 
 
 // A chunk is staged in 128 / PS pieces of PS positions (the contraction over positions is a plain sum): the
 // smaller the piece, the smaller the LDS tiles and the prefetch registers, but the more barriers per chunk.
-// Measured on MI355X (B=4, S=16384, NH=8, 256/512), forward / backward scan in ms:
-//   four waves per 128 x 128 tile, one workgroup per CU (one wave per SIMD)      0.63 / 0.54
-//   four waves, register cap for two workgroups per CU (backward: 78 KB LDS)     -    / 0.46
-//   four waves, half-chunk pieces so that the forward fits twice per CU          0.66 / 0.55
-//   eight waves per tile (64 x 32 per wave), one workgroup per CU                0.46 / 0.41   <- scan_kernel
-//   eight waves, two workgroups per CU (128 registers per lane)                  -    / 0.45
-//   n recurrence shared out among the column tiles by lane masks / run by every column tile    0.51 / -    (0.48 used)
-//   rows moved from global memory straight into LDS (global_load_lds_dwordx4 into a ring of four 64-position stages,
-//   three stages ahead, XOR-swizzled tiles, one barrier per stage, rows scaled in place)   0.44 / 0.45
-//     (bit-equal results; with parts switched off: loads alone 0.22, state stores 0.05, matrix work 0.10, in-place
-//      scaling 0.04, barriers 0.04 -- the parts add up instead of overlapping, and waiting less for the loads does
-//      not change the time)
-//   two LDS buffers and two register sets, one barrier per chunk: the rows of chunk c+1 are scaled and written into
-//   one buffer while chunk c is multiplied out of the other, chunk c+3 is requested meanwhile (unpadded swizzled
-//   tiles, 141 KB)                                                0.37 / 0.36 without the n recurrence, 0.44 with it
-//     (bit-equal states.  Per chunk a CU spends about 1500 cycles on LDS traffic, 1000 per SIMD on matrix
-//      instructions and 1000 per SIMD on the conversion arithmetic of the staging; with two waves per SIMD these
-//      mostly add up, whatever the order they are issued in: 2.2 us per chunk even at B = 1, where nothing else
-//      uses the memory system)
-//   the same two buffers, but sixteen waves in two roles: eight producer waves fetch, scale and stage the rows,
-//   eight consumer waves do the fragment reads and matrix instructions; the normaliser recurrence as three more
-//   operand columns on the consumers' matrix pipe                  0.33 / 0.29   <- used when no last state is returned
+// scan_kernel: eight waves per 128 x 128 tile (64 x 32 per wave), one workgroup per CU.  scan_roles_kernel: two LDS
+// buffers and sixteen waves in two roles -- eight producer waves fetch, scale and stage the rows of chunk c+1 while
+// eight consumer waves do the fragment reads and matrix instructions of chunk c (one barrier per chunk); the
+// normaliser recurrence rides as three more operand columns on the consumers' matrix pipe.
 // What pays is more instruction streams per SIMD inside the same workgroup: the phases of a chunk (staging, state
 // emission, matrix work) are serial per wave; two waves per SIMD overlap one's LDS and conversion latencies with the
 // other's matrix instructions, and four waves in two roles keep the conversion arithmetic and the matrix
