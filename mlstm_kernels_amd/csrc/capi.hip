@@ -86,12 +86,15 @@ const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, h
     return mlstm::launch_stream_hv(a, BH, is_dv, st);
   return mlstm::launch_par_hv(a, BH, is_dv, st);
 }
-// dQ / dK launch: the streaming kernel under the same rule
+// dQ / dK launch.  MLSTM_PATH_STREAM: the window kernel (state stride 2) or the streaming kernel per chunk and
+// gradient (other strides); MLSTM_PATH_AUTO: the window kernel where the shape allows, else the tiled pair kernel
+// (faster than the per-chunk streaming kernel); MLSTM_PATH_SPLIT: the tiled pair kernel
 const char* launch_qk(int path, const mlstm::ParQkArgs& a, int BH, hipStream_t st) {
   if (path == MLSTM_PATH_STREAM && !mlstm::stream_qk_supported(a))
     return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 without head norm only";
-  // (MLSTM_PATH_AUTO keeps the tiled pair kernel: it is the faster one of the two as measured today)
-  if (path == MLSTM_PATH_STREAM && mlstm::stream_qk_supported(a)) return mlstm::launch_stream_qk(a, BH, st);
+  if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::window_qk_supported(a))
+    return mlstm::launch_window_qk(a, BH, st);
+  if (path == MLSTM_PATH_STREAM) return mlstm::launch_stream_qk(a, BH, st);
   return mlstm::launch_par_qk_pair(a, BH, st);
 }
 const char* check_dims(int B, int NH, int S, int DHQK, int DHHV) {

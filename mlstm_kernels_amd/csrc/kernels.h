@@ -131,6 +131,8 @@ bool fused_hv_supported(int DHQK, int DHHV);
 const char* launch_fused_hv(const FusedHvArgs& a, int BH, bool is_dv, hipStream_t stream);
 const char* launch_par_qk_pair(const ParQkArgs& a, int BH, hipStream_t stream);
 // streaming (persistent, producer / consumer waves) form of the same launch for the shapes it supports
+bool window_qk_supported(const ParQkArgs& a);
+const char* launch_window_qk(const ParQkArgs& a, int BH, hipStream_t stream);
 bool stream_qk_supported(const ParQkArgs& a);
 const char* launch_stream_qk(const ParQkArgs& a, int BH, hipStream_t stream);
 int par_qk_head_tile(int DHQK);  // head-dimension rows per workgroup of the dQ/dK kernel
