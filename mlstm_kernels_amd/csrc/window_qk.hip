@@ -16,14 +16,17 @@
 //   * Three phases per window, all with a static step structure (NV = DHHV / 32):
 //       S  NV steps  [dH rows x 32 value columns | V rows x 32 value columns]      scores of all 36 blocks, then gating
 //       Q  NV steps  [C fragments of 32 value columns | dH rows x 32 columns]      Out^T += C dH^T  (256 x 256 tile)
-//           4 steps  [64 K rows x 256 head-dim entries]                            Out^T += K^T P^T ; dQ rows leave
-//       K  NV steps  [dC fragments | V rows],  4 steps [64 Q rows]                 the same for dK (P read transposed)
-//     A window moves 3 * DHHV + 256 KB through the CU (1792 KB at DHHV = 512) where its four chunk-and-gradient items
+//           4 steps  [64 K rows x 256 head-dim entries]                            Out^T += K^T P^T
+//           4 steps  [64 Q rows]                                                   row dots q . dQ; dQ rows leave
+//       K  NV steps  [dC fragments | V rows],  4 steps [64 Q rows], 4 steps [64 K rows]   the same for dK (P read
+//                                                                                  transposed)
+//     A window moves 3 * DHHV + 512 KB through the CU (2048 KB at DHHV = 512) where its four chunk-and-gradient items
 //     take 2944 KB in stream_qk.hip, and multiplies every score block once instead of twice.
 //   * A consumer wave owns 64 head-dim rows x four 32-position blocks of alternating parity (128 accumulator
-//     registers); the causal structure then loads both parities nearly alike.  Results leave through a private
-//     2 KB staging tile per wave: eight positions at a time the fp32 accumulators are turned into row order, meet
-//     the q (k) rows for the gate-gradient row dots, are rounded and stored as full 128-byte lines.
+//     registers); the causal structure then loads both parities nearly alike.  The q (k) rows of the gate-gradient
+//     row dots come through the ring like every other operand (fetched by the consumers themselves they cost a
+//     memory latency per handful of positions); the rounded results pass through a private 2 KB staging tile per
+//     wave into row order and are stored as full 128-byte lines.
 // Supported: state stride 2, DHQK = 256, DHHV a multiple of 64, S a multiple of 256.
 #include <type_traits>
 
@@ -51,7 +54,7 @@ constexpr int kWqSlot = 32768;                    // bytes per ring slot = per s
 constexpr int kWqPOfs = 2 * kWqSlot;              // P: 36 blocks of 32 x 32 (2 KB each, 64-byte rows, swizzled)
 constexpr int kWqVecOfs = kWqPOfs + 36 * 2048;    // u[256], w[256], lqr[256] (fp32)
 constexpr int kWqRedOfs = kWqVecOfs + 3 * 1024;   // [4][256] row-dot partials per 64-row block of the head dimension
-constexpr int kWqStgOfs = kWqRedOfs + 4 * 1024;   // [8 waves][8 rows][64 fp32] staging tiles
+constexpr int kWqStgOfs = kWqRedOfs + 4 * 1024;   // [8 waves][16 rows][64 elements] staging tiles
 constexpr int kWqSmem = kWqStgOfs + 8 * 2048;
 static_assert(kWqSmem <= 160 * 1024, "LDS budget of one CU");
 
@@ -163,29 +166,45 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
       const uint32_t zrow = pl >> 5, zun = pl & 31;
       const uint32_t zdu = zrow * 32 + (zun ^ (2 * (zrow & 3)));
       const uint32_t zg = (t0 + zrow) * (DHQK * 2) + zun * 16;
+      // (every loop works on its own opaque copy of the offsets: addresses shared between two loops would otherwise be
+      // kept, and spilled, across everything in between)
+#define WQ_ROWS(bA_, bB_)                                                                                            \
+  {                                                                                                                  \
+    const uint32_t zz = (uint32_t)opaque((int)zg);                                                                   \
+    for (int z = 0; z < 4; z += 2) {                                                                                 \
+      WQ_PROC(0, bA_, zz + z * 32768, 4096, bB_, zz + z * 32768 + 16384, 4096, zdu, 1024 + zdu)                      \
+      WQ_PROC(1, bA_, zz + (z + 1) * 32768, 4096, bB_, zz + (z + 1) * 32768 + 16384, 4096, zdu, 1024 + zdu)          \
+    }                                                                                                                \
+  }
       // ---- phase S: dH rows | V rows
-      for (int w = 0; w < NV; w += 2) {
-        WQ_PROC(0, dH_b, xg + w * 64, xstep, V_b, xg + w * 64, xstep, xdu, 1024 + xdu)
-        WQ_PROC(1, dH_b, xg + (w + 1) * 64, xstep, V_b, xg + (w + 1) * 64, xstep, xdu, 1024 + xdu)
+      {
+        const uint32_t xx = (uint32_t)opaque((int)xg);
+        for (int w = 0; w < NV; w += 2) {
+          WQ_PROC(0, dH_b, xx + w * 64, xstep, V_b, xx + w * 64, xstep, xdu, 1024 + xdu)
+          WQ_PROC(1, dH_b, xx + (w + 1) * 64, xstep, V_b, xx + (w + 1) * 64, xstep, xdu, 1024 + xdu)
+        }
       }
-      // ---- phase Q: C fragments | dH rows, then the K rows
-      for (int w = 0; w < NV; w += 2) {
-        WQ_PROC(0, C_b, (uint32_t)w * 16384 + pl * 16, 4096, dH_b, xg + w * 64, xstep, cdu, 1024 + xdu)
-        WQ_PROC(1, C_b, (uint32_t)(w + 1) * 16384 + pl * 16, 4096, dH_b, xg + (w + 1) * 64, xstep, cdu, 1024 + xdu)
+      // ---- phase Q: C fragments | dH rows, then the K rows (products) and the Q rows (row dots)
+      {
+        const uint32_t xx = (uint32_t)opaque((int)xg), cc = (uint32_t)opaque((int)(pl * 16));
+        for (int w = 0; w < NV; w += 2) {
+          WQ_PROC(0, C_b, (uint32_t)w * 16384 + cc, 4096, dH_b, xx + w * 64, xstep, cdu, 1024 + xdu)
+          WQ_PROC(1, C_b, (uint32_t)(w + 1) * 16384 + cc, 4096, dH_b, xx + (w + 1) * 64, xstep, cdu, 1024 + xdu)
+        }
       }
-      for (int z = 0; z < 4; z += 2) {
-        WQ_PROC(0, K_b, zg + z * 32768, 4096, K_b, zg + z * 32768 + 16384, 4096, zdu, 1024 + zdu)
-        WQ_PROC(1, K_b, zg + (z + 1) * 32768, 4096, K_b, zg + (z + 1) * 32768 + 16384, 4096, zdu, 1024 + zdu)
+      WQ_ROWS(K_b, K_b)
+      WQ_ROWS(Q_b, Q_b)
+      // ---- phase K: dC fragments | V rows, then the Q rows (products) and the K rows (row dots)
+      {
+        const uint32_t xx = (uint32_t)opaque((int)xg), cc = (uint32_t)opaque((int)(pl * 16));
+        for (int w = 0; w < NV; w += 2) {
+          WQ_PROC(0, dC_b, (uint32_t)w * 16384 + cc, 4096, V_b, xx + w * 64, xstep, cdu, 1024 + xdu)
+          WQ_PROC(1, dC_b, (uint32_t)(w + 1) * 16384 + cc, 4096, V_b, xx + (w + 1) * 64, xstep, cdu, 1024 + xdu)
+        }
       }
-      // ---- phase K: dC fragments | V rows, then the Q rows
-      for (int w = 0; w < NV; w += 2) {
-        WQ_PROC(0, dC_b, (uint32_t)w * 16384 + pl * 16, 4096, V_b, xg + w * 64, xstep, cdu, 1024 + xdu)
-        WQ_PROC(1, dC_b, (uint32_t)(w + 1) * 16384 + pl * 16, 4096, V_b, xg + (w + 1) * 64, xstep, cdu, 1024 + xdu)
-      }
-      for (int z = 0; z < 4; z += 2) {
-        WQ_PROC(0, Q_b, zg + z * 32768, 4096, Q_b, zg + z * 32768 + 16384, 4096, zdu, 1024 + zdu)
-        WQ_PROC(1, Q_b, zg + (z + 1) * 32768, 4096, Q_b, zg + (z + 1) * 32768 + 16384, 4096, zdu, 1024 + zdu)
-      }
+      WQ_ROWS(Q_b, Q_b)
+      WQ_ROWS(K_b, K_b)
+#undef WQ_ROWS
     }
     // ---- drain: the last two slabs go to LDS, then the barriers of the consumers' last steps and of the final row dots
     if (L > 0) {
@@ -438,62 +457,58 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
           }
         }
 
-        // ---- results: eight positions at a time the fp32 accumulators pass through the wave's staging tile into row
-        // order; there they meet the x rows (q for dQ, k for dK) for the row dots sum_d x Out (taken from the fp32
-        // values: they feed a suffix sum over the whole sequence, where the rounding noise of 16-bit outputs would
-        // add up), are rounded and leave as full lines.  Everything here is private to the wave.
-        {
-          // row-order role of a lane: position row8 of the round, head-dim entries 8 dg .. 8 dg + 7 of the wave's 64
-          const char* const Xb = (const char*)(dk ? a.K : a.Q) + ((size_t)bh * S + (size_t)c0 * kChunk) * (DHQK * 2);
-          char* const Ob = (char*)(dk ? a.Out2 : a.Out) + ((size_t)bh * S + (size_t)c0 * kChunk) * (DHQK * 2);
-          const uint32_t lofs = (uint32_t)((opaque(lane) >> 3) * (DHQK * 2) + 128 * di + 16 * (opaque(lane) & 7));
-          u32x4 xq[2];
+        // ---- results, 64 positions per step: the x rows (q for dQ, k for dK) of those positions arrive as one more
+        // slab; every wave owns one 32-position block of them.  Row dots sum_d x Out from the fp32 accumulators (they
+        // feed a suffix sum over the whole sequence, where the rounding noise of 16-bit outputs would add up); then
+        // the rounded values pass, 16 positions at a time, through the wave's private staging tile into row order and
+        // leave as full 128-byte lines.
+        char* const Ob = (char*)(dk ? a.Out2 : a.Out) + ((size_t)bh * S + (size_t)c0 * kChunk) * (DHQK * 2);
 #pragma unroll
-          for (int pf = 0; pf < 2; ++pf)   // rounds 0 and 1 are the first two quarters of block nb = 0
-            xq[pf] = *(const u32x4*)(Xb + (lofs + (uint32_t)((32 * par + 8 * pf) * (DHQK * 2))));
+        for (int z = 0; z < 4; ++z) {
+          __syncthreads();
+          const unsigned char* const Xs = next_slab();
+          const int le = opaque(lane);
+          const int r = le & 31, h = le >> 5;
+          {
+            const int row = 32 * par + r;
+            const unsigned char* const xrow = Xs + row * 512 + 8 * h;
+            const int sw = 2 * (row & 3);
+            float part = 0.f;
 #pragma unroll
-          for (int nb = 0; nb < 4; ++nb)
+            for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int n0 = 32 * (2 * nb + par) + 8 * q;   // first position of the round
-              const int le = opaque(lane);
-              const int r = le & 31, h = le >> 5;
-              const int row8 = le >> 3, dg = le & 7;
-              if ((r >> 3) == q) {
-                const int row = r & 7;
-#pragma unroll
-                for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-                  for (int g4 = 0; g4 < 4; ++g4) {
-                    const int un = 8 * mb + 2 * g4 + h;
-                    f32x4 v = {acc[mb][nb][4 * g4 + 0], acc[mb][nb][4 * g4 + 1], acc[mb][nb][4 * g4 + 2],
-                               acc[mb][nb][4 * g4 + 3]};
-                    *(f32x4*)(stg + row * 256 + ((un ^ (2 * row)) * 16)) = v;
-                  }
+              for (int g4 = 0; g4 < 4; ++g4) {
+                const uint2 xv = *(const uint2*)(xrow + (((8 * di + 4 * mb + g4) ^ sw) * 16));
+                part += acc[mb][z][4 * g4 + 0] * lo2<F16>(xv.x);
+                part += acc[mb][z][4 * g4 + 1] * hi2<F16>(xv.x);
+                part += acc[mb][z][4 * g4 + 2] * lo2<F16>(xv.y);
+                part += acc[mb][z][4 * g4 + 3] * hi2<F16>(xv.y);
               }
-              __builtin_amdgcn_wave_barrier();
-              const f32x4 v0 = *(const f32x4*)(stg + row8 * 256 + (((2 * dg) ^ (2 * row8)) * 16));
-              const f32x4 v1 = *(const f32x4*)(stg + row8 * 256 + (((2 * dg + 1) ^ (2 * row8)) * 16));
-              __builtin_amdgcn_wave_barrier();
-              const u32x4 xv = xq[q & 1];
-              {
-                // the x rows of the round after the next one
-                const int nb2 = q < 2 ? nb : nb + 1, q2 = (q + 2) & 3;
-                if (nb2 < 4)
-                  xq[q & 1] = *(const u32x4*)(Xb + (lofs + (uint32_t)((32 * (2 * nb2 + par) + 8 * q2) * (DHQK * 2))));
-              }
-              float part = v0[0] * lo2<F16>(xv[0]) + v0[1] * hi2<F16>(xv[0]);
-              part += v0[2] * lo2<F16>(xv[1]) + v0[3] * hi2<F16>(xv[1]);
-              part += v1[0] * lo2<F16>(xv[2]) + v1[1] * hi2<F16>(xv[2]);
-              part += v1[2] * lo2<F16>(xv[3]) + v1[3] * hi2<F16>(xv[3]);
-              part += __shfl_xor(part, 1);
-              part += __shfl_xor(part, 2);
-              part += __shfl_xor(part, 4);
-              if (dg == 0) red[di * 256 + n0 + row8] = part;
-              const u32x4 ov = {pack2<F16>(v0[0], v0[1]), pack2<F16>(v0[2], v0[3]), pack2<F16>(v1[0], v1[1]),
-                                pack2<F16>(v1[2], v1[3])};
-              __builtin_nontemporal_store(ov, (u32x4*)(Ob + (lofs + (uint32_t)(n0 * (DHQK * 2)))));
+            part += __shfl_xor(part, 32);
+            if (h == 0) red[di * 256 + 64 * z + row] = part;
+          }
+          const uint32_t lofs = (uint32_t)((le >> 3) * (DHQK * 2) + 128 * di + 16 * (le & 7));
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            if ((r >> 4) == q) {
+              const int row = r & 15;
+#pragma unroll
+              for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4)
+                  *(uint2*)(stg + row * 128 + (((4 * mb + g4) ^ (row & 7)) * 16) + 8 * h) =
+                      make_uint2(pack2<F16>(acc[mb][z][4 * g4 + 0], acc[mb][z][4 * g4 + 1]),
+                                 pack2<F16>(acc[mb][z][4 * g4 + 2], acc[mb][z][4 * g4 + 3]));
             }
+            __builtin_amdgcn_wave_barrier();
+            const int row8 = le >> 3, un = le & 7;
+            const u32x4 o0 = *(const u32x4*)(stg + row8 * 128 + ((un ^ row8) * 16));
+            const u32x4 o1 = *(const u32x4*)(stg + (row8 + 8) * 128 + ((un ^ row8) * 16));
+            __builtin_amdgcn_wave_barrier();
+            const uint32_t n0 = (uint32_t)(64 * z + 32 * par + 16 * q);
+            __builtin_nontemporal_store(o0, (u32x4*)(Ob + (lofs + n0 * (DHQK * 2))));
+            __builtin_nontemporal_store(o1, (u32x4*)(Ob + (lofs + (n0 + 8) * (DHQK * 2))));
+          }
         }
         pending = dk ? 2 : 1;
       };

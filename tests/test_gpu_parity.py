@@ -32,11 +32,13 @@ DEV = "cuda"
 _VARIANT = {"kernel_path": "auto", "chunk_size_intra": None}
 
 
-@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "stream-1", "stream-2", "stream-4", "fused-1"])
+@pytest.fixture(autouse=True, params=["split-1", "split-2", "split-4", "stream-1", "stream-2", "stream-4", "auto-2", "fused-1"])
 def kernel_variant(request):
     """Every test runs once per kernel variant of the chunkwise passes: the split path (state scan + chunk-parallel
     kernels) with a chunk state kept every 1, 2 or 4 chunks, the stream path (the same scans, chunk-parallel kernels
-    as persistent workgroups with producer and consumer waves; shapes it does not support are skipped), and the fused
+    as persistent workgroups with producer and consumer waves; shapes it does not support are skipped; at stride 2
+    dQ and dK come from the window kernel), the library's own choice at its default stride ("auto-2": streaming H / dV
+    and the window dQ / dK kernel wherever each supports the shape, the tiled kernels elsewhere), and the fused
     path (sequential kernels with a register-resident state; head dimensions it does not support are skipped; stride
     1, so that all its kernels group the products the same way -- the fused path with other strides is part of the
     randomised sweep)."""
@@ -589,6 +591,10 @@ def _fwbw_case(B, NH, S, DQK, DHV, siging=False, normalize=True, init=False, dcl
     dict(B=1, NH=2, S=256, DQK=64, DHV=64, siging=True, init=True, seed=14, dtype=torch.float16),
     dict(B=1, NH=2, S=400, DQK=192, DHV=64, L=16, init=True, seed=15, last=False, dtype=torch.float16),
     dict(B=1, NH=1, S=384, DQK=896, DHV=128, init=True, seed=16, dtype=torch.float16),
+    # shapes of the window dQ / dK kernel (DHQK = 256, windows of 256 positions) beside the benchmark's value width
+    dict(B=1, NH=3, S=768, DQK=256, DHV=192, init=True, dcl=True, seed=17),
+    dict(B=2, NH=2, S=512, DQK=256, DHV=1024, seed=18, last=False, dtype=torch.float16),
+    dict(B=1, NH=5, S=512, DQK=256, DHV=128, siging=True, init=True, seed=19),
 ])
 def test_chunkwise_fwbw_small(kw):
     _fwbw_case(**kw)
