@@ -673,7 +673,7 @@ def test_chunkwise_every_element_within_tolerance_of_the_rounding_emulation(kw, 
     track_n = not (siging and not normalize)
     _, qb, kb, vb, ib, fb, c0f, n0f, m0f = X._prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
     n_kernel = torch.empty(B, NH, S, dtype=torch.float32, device=DEV)
-    path = _lib.PATH_STREAM if kernel_variant.startswith("stream") else _lib.PATH_SPLIT
+    path = _lib.path_code(kernel_variant.split("-")[0])   # the same forward kernels as the call above
     X._fw_launch(qb, kb, vb, ib, fb, c0f, n0f, m0f, 1e-6, siging, normalize, False, False, path, stride,
                  n_out=n_kernel)
     rnd = R.rounder(dtype)
