@@ -60,12 +60,16 @@ const char* mlstm_hip_last_error(void);
  * path: kernel selection for the value-column side of the passes (H forward, dV backward).  No counterpart in the
  * reference, whose Triton kernels are always the two-kernel form, recurrent_fw_C followed by parallel_fw_Hintra
  * (mlstm_kernels/torch/chunkwise/triton_xl_chunk/fw.py:20-136).
- *   MLSTM_PATH_AUTO  : the fastest one for the shape as measured on MI355X (stream where it applies, else split)
+ *   MLSTM_PATH_AUTO  : the fastest one for the shape as measured on MI355X: the streaming H / dV kernels where the
+ *                      conditions of MLSTM_PATH_STREAM hold, the window dQ / dK kernel (windows of two chunks that
+ *                      share a kept state) at state_stride 2 with DHQK = 256, DHHV a multiple of 64 and S a multiple
+ *                      of 256, the kernels of MLSTM_PATH_SPLIT for everything else
  *   MLSTM_PATH_SPLIT : state scan + chunk-parallel kernel over materialised chunk states
  *   MLSTM_PATH_STREAM: the split form with the chunk-parallel kernels as persistent workgroups whose waves are split
  *                      into producers (global memory -> LDS, several slabs in flight) and consumers (matrix
  *                      instructions); DHQK = 256, DHHV a multiple of 512, S a multiple of 128, no head norm: other
- *                      shapes are rejected.  Same workspaces as MLSTM_PATH_SPLIT.
+ *                      shapes are rejected.  dQ / dK: the window kernel under the conditions above, else a
+ *                      streaming kernel per chunk and gradient.  Same workspaces as MLSTM_PATH_SPLIT.
  *   MLSTM_PATH_FUSED : one sequential kernel per pass, state slice resident in registers (DHQK = 128 or 256 only:
  *                      other head dimensions are rejected)
  *
