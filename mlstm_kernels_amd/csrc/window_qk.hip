@@ -55,7 +55,8 @@ constexpr int kWqPOfs = 2 * kWqSlot;              // P: 36 blocks of 32 x 32 (2 
 constexpr int kWqVecOfs = kWqPOfs + 36 * 2048;    // u[256], w[256], lqr[256] (fp32)
 constexpr int kWqRedOfs = kWqVecOfs + 3 * 1024;   // [4][256] row-dot partials per 64-row block of the head dimension
 constexpr int kWqStgOfs = kWqRedOfs + 4 * 1024;   // [8 waves][16 rows][64 elements] staging tiles
-constexpr int kWqSmem = kWqStgOfs + 8 * 2048;
+constexpr int kWqCsOfs = kWqStgOfs + 8 * 2048;    // [256] column scale of the inter-chunk part of the running phase
+constexpr int kWqSmem = kWqCsOfs + 1024;
 static_assert(kWqSmem <= 160 * 1024, "LDS budget of one CU");
 
 // the blocks (tb, jb) of the lower triangle a consumer wave computes in phase S: up to five, at most two distinct tb
@@ -93,6 +94,7 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
   float* const wvec = uvec + 256;                      // [256] w_j
   float* const lqr = wvec + 256;                       // [256] log2(rho_t / sqrt(DHQK))
   float* const red = (float*)(smem_raw + kWqRedOfs);
+  float* const csv = (float*)(smem_raw + kWqCsOfs);
 
   const int lane = threadIdx.x & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
@@ -331,24 +333,18 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
       // ============================================================================ phases Q (dQ) and K (dK)
       auto run_phase = [&](auto DKT) {
         constexpr bool dk = decltype(DKT)::value;
-        // column scale of the inter-chunk part per position block (requested now, used after the value pass)
-        float csr[4];
-        {
-          const int r = opaque(lane) & 31;
-          float xs;
-          if (dk) xs = __expf(graw[c0 + 1] + mst[c0 + 1] - mst[c0 + 2]);   // keys of c0 see dC through chunk c1
-          else xs = __expf(g01 + mst[c0] - mst[c0 + 1]);                   // positions of c1 see C through chunk c0
-#pragma unroll
-          for (int nb = 0; nb < 4; ++nb) {
-            const int n = 32 * (2 * nb + par) + r;
-            const size_t gi = gofs + n;
-            const bool far = dk ? n < 128 : n >= 128;
-            if (dk) {
-              csr[nb] = a.g.abar[gi] * (far ? xs : 1.f);
-            } else {
-              const float rh = a.use_nrow ? 1.f / (a.nrow[gi] + a.eps) : 1.f;
-              csr[nb] = a.g.bbar[gi] * a.qk_scale * rh * (far ? xs : 1.f);
-            }
+        // column scale of the inter-chunk part: requested now by one thread per position, parked in LDS after the first
+        // step of the value pass, used after its last one (registers are what this kernel is short of)
+        float csn = 0.f;
+        if (tid < 256) {
+          const size_t gi = gofs + tid;
+          if (dk) {
+            const float xs = __expf(graw[c0 + 1] + mst[c0 + 1] - mst[c0 + 2]);   // keys of c0 see dC through chunk c1
+            csn = a.g.abar[gi] * (tid < 128 ? xs : 1.f);
+          } else {
+            const float xs = __expf(g01 + mst[c0] - mst[c0 + 1]);                // positions of c1 see C through chunk c0
+            const float rh = a.use_nrow ? 1.f / (a.nrow[gi] + a.eps) : 1.f;
+            csn = a.g.bbar[gi] * a.qk_scale * rh * (tid >= 128 ? xs : 1.f);
           }
         }
 #pragma unroll
@@ -364,7 +360,10 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
         for (int w = 0; w < NV; ++w) {
           __syncthreads();
           const unsigned char* const Cf = next_slab();
-          if (w == 0) finish_rowdots();
+          if (w == 0) {
+            finish_rowdots();
+            if (tid < 256) csv[tid] = csn;   // (read after the last step of this loop: NV - 1 >= 1 barriers later)
+          }
           const unsigned char* const Xn = Cf + 16384;
           const int le = opaque(lane);
           const int r = le & 31, h = le >> 5;
@@ -399,9 +398,11 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
         // column scale of the inter-chunk part (kept apart from the matrix instructions around it)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb)
+        for (int nb = 0; nb < 4; ++nb) {
+          const float cs = csv[32 * (2 * nb + par) + (opaque(lane) & 31)];
 #pragma unroll
-          for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= csr[nb];
+          for (int mb = 0; mb < 2; ++mb) acc[mb][nb] *= cs;
+        }
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- Out^T += Z^T P'^T over the 256 positions of the window, 64 rows of Z per slab (Z = K for dQ with
