@@ -67,8 +67,8 @@ const char* mlstm_hip_last_error(void);
  *   MLSTM_PATH_SPLIT : state scan + chunk-parallel kernel over materialised chunk states
  *   MLSTM_PATH_STREAM: the split form with the chunk-parallel kernels as persistent workgroups whose waves are split
  *                      into producers (global memory -> LDS, several slabs in flight) and consumers (matrix
- *                      instructions); DHQK = 256, DHHV a multiple of 512, S a multiple of 128, no head norm: other
- *                      shapes are rejected.  dQ / dK: the window kernel under the conditions above, else a
+ *                      instructions); DHQK = 256, DHHV a multiple of 512 (exactly 512 with a head norm), S a
+ *                      multiple of 128: other shapes are rejected.  dQ / dK: the window kernel under the conditions above, else a
  *                      streaming kernel per chunk and gradient.  Same workspaces as MLSTM_PATH_SPLIT.
  *   MLSTM_PATH_FUSED : one sequential kernel per pass, state slice resident in registers (DHQK = 128 or 256 only:
  *                      other head dimensions are rejected)

@@ -81,7 +81,7 @@ const char* check_options(int path, int state_stride, int DHQK, int DHHV) {
 // shape is one it supports, otherwise the tiled kernel
 const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, hipStream_t st) {
   if (path == MLSTM_PATH_STREAM && !mlstm::stream_hv_supported(a))
-    return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 without head norm only";
+    return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 only (with a head norm: DHHV = 512)";
   if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::stream_hv_supported(a))
     return mlstm::launch_stream_hv(a, BH, is_dv, st);
   return mlstm::launch_par_hv(a, BH, is_dv, st);
@@ -91,7 +91,7 @@ const char* launch_hv(int path, const mlstm::ParHvArgs& a, int BH, bool is_dv, h
 // (faster than the per-chunk streaming kernel); MLSTM_PATH_SPLIT: the tiled pair kernel
 const char* launch_qk(int path, const mlstm::ParQkArgs& a, int BH, hipStream_t st) {
   if (path == MLSTM_PATH_STREAM && !mlstm::stream_qk_supported(a))
-    return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 without head norm only";
+    return "the stream kernel path supports DHQK = 256, DHHV % 512 == 0, S % 128 == 0 only (with a head norm: DHHV = 512)";
   if ((path == MLSTM_PATH_STREAM || path == MLSTM_PATH_AUTO) && mlstm::window_qk_supported(a))
     return mlstm::launch_window_qk(a, BH, st);
   if (path == MLSTM_PATH_STREAM) return mlstm::launch_stream_qk(a, BH, st);

@@ -70,8 +70,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 }  // namespace
 
-template <bool IS_DV, bool F16>
+// NORM (forward, DHHV = 512: a work item then holds complete rows of H): the multi-head layer / rms norm over the value
+// columns is applied when the rows are rounded, as an affine map of the accumulators.
+template <bool IS_DV, bool F16, bool NORM = false>
 __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items, int n_rounds) {
+  static_assert(!(IS_DV && NORM), "the head norm belongs to the forward");
   constexpr int DHQK = 256;
   constexpr int QS = DHQK + 8;   // resident rows [128][DHQK] and score-operand slabs [64][DHQK], fragment order
   constexpr int VS = 512 + 16;   // value-operand slab: 32 rows x 512 value columns, row-major
@@ -94,6 +97,7 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
   float* const orho = ovec + 64;               // [64] dV: rho_t of the source half
   float* const denq = orho + 64;               // [128] forward: bbar_t / sqrt(d) * (q_t . n_prev), the inter-chunk part of the denominator
   float* const mcv = denq + 128;               // [128] forward: combined stabiliser of the item's positions
+  float* const nst = mcv + 128;                // NORM: [4][2][128] sum and sum of squares of a row over each wave's 128 columns
   constexpr uint32_t kRing0Off = 128 * QS * 2, kRing1Off = kRing0Off + (SLOT + 128 * PSS) * 2;
 
   const int lane = threadIdx.x & 63;
@@ -278,11 +282,30 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
     const int r = le & 31, h = le >> 5;                                                                              \
     constexpr int SR = 32 * (NMB_) + 8; /* staging row */                                                            \
     uint16_t* const stg = (STG_);                                                                                    \
-    const float iv = IS_DV ? 1.f : inv[64 * pi + 32 * NB + r];                                                       \
+    float iv = IS_DV ? 1.f : inv[64 * pi + 32 * NB + r];                                                             \
+    float sh = 0.f;                                                                                                  \
+    if constexpr (NORM) {                                                                                            \
+      /* x = acc * iv is the row of H; mean and variance over its 512 columns from the four waves' sums */            \
+      const int t_ = 64 * pi + 32 * NB + r;                                                                          \
+      const float t1_ = (nst[t_] + nst[256 + t_]) + (nst[512 + t_] + nst[768 + t_]);                                 \
+      const float t2_ = (nst[128 + t_] + nst[384 + t_]) + (nst[640 + t_] + nst[896 + t_]);                           \
+      const float ex_ = t1_ * iv * (1.f / 512.f), ex2_ = t2_ * iv * iv * (1.f / 512.f);                              \
+      const float mean_ = a.head_norm == 1 ? ex_ : 0.f;                                                              \
+      const float rstd_ = rsqrtf(fmaxf(ex2_ - mean_ * mean_, 0.f) + a.norm_eps);                                     \
+      if (ci == 0 && h == 0) {                                                                                       \
+        const size_t tg_ = (size_t)prev.bh * S + (size_t)prev.c * kChunk + t_;                                       \
+        a.norm_mean[tg_] = mean_;                                                                                    \
+        a.norm_rstd[tg_] = rstd_;                                                                                    \
+      }                                                                                                              \
+      iv *= rstd_;                                                                                                   \
+      sh = -mean_ * rstd_;                                                                                           \
+    }                                                                                                                \
     _Pragma("unroll") for (int mb = 0; mb < (NMB_); ++mb) _Pragma("unroll") for (int g4 = 0; g4 < 4; ++g4) {         \
       *(uint2*)(stg + r * SR + 32 * mb + 8 * g4 + 4 * h) =                                                           \
-          make_uint2(pack2<F16>(acc[(MB0_) + mb][NB][4 * g4 + 0] * iv, acc[(MB0_) + mb][NB][4 * g4 + 1] * iv),       \
-                     pack2<F16>(acc[(MB0_) + mb][NB][4 * g4 + 2] * iv, acc[(MB0_) + mb][NB][4 * g4 + 3] * iv));      \
+          make_uint2(pack2<F16>(__builtin_fmaf(acc[(MB0_) + mb][NB][4 * g4 + 0], iv, sh),                            \
+                                __builtin_fmaf(acc[(MB0_) + mb][NB][4 * g4 + 1], iv, sh)),                           \
+                     pack2<F16>(__builtin_fmaf(acc[(MB0_) + mb][NB][4 * g4 + 2], iv, sh),                            \
+                                __builtin_fmaf(acc[(MB0_) + mb][NB][4 * g4 + 3], iv, sh)));                          \
     }                                                                                                                \
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                                           \
     __builtin_amdgcn_wave_barrier();                                                                                 \
@@ -497,6 +520,29 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb) mfma32<F16>(acc[mb][nb], A[mb], B[nb]);
             }
+            if constexpr (NORM) {
+              // ---- sums over this wave's 128 columns of every row, from the finished accumulators
+              if (own && kh == 1 && vi == 1) {
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) {
+                  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                      const float x = acc[mb][nb][i];
+                      s1 += x;
+                      s2 = __builtin_fmaf(x, x, s2);
+                    }
+                  s1 += __shfl_xor(s1, 32);
+                  s2 += __shfl_xor(s2, 32);
+                  if (h == 0) {
+                    nst[ci * 256 + 64 * pi + 32 * nb + r] = s1;
+                    nst[ci * 256 + 128 + 64 * pi + 32 * nb + r] = s2;
+                  }
+                }
+              }
+            }
             // ---- forward: denominators, once all row sums of the own chunk are there (it is the last source chunk)
             if (!IS_DV && own && kh == 1 && vi == 1) {
               const int td = opaque(tid);
@@ -538,7 +584,9 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
 }
 
 bool stream_hv_supported(const ParHvArgs& a) {
-  return a.DHQK == 256 && a.DHHV % 512 == 0 && a.S % kChunk == 0 && a.head_norm == 0;
+  // with the fused head norm a work item must hold complete rows: one group of 512 value columns
+  const bool norm_ok = a.head_norm == 0 || (a.DHHV == 512 && a.norm_mean != nullptr && a.norm_rstd != nullptr);
+  return a.DHQK == 256 && a.DHHV % 512 == 0 && a.S % kChunk == 0 && norm_ok;
 }
 
 namespace {
@@ -554,10 +602,11 @@ int device_cu_count() {
   return cached[dev];
 }
 
-template <bool IS_DV, bool F16>
+template <bool IS_DV, bool F16, bool NORM = false>
 const char* launch_stream_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
   constexpr int QS = 256 + 8, PSS = 72, SLOT = 64 * QS;
-  const size_t smem = (size_t)(128 * QS + 128 * PSS + 2 * SLOT) * 2 + (size_t)(4 * 128 + 128 + 256 + 64 + 64 + 128 + 128) * 4;
+  const size_t smem = (size_t)(128 * QS + 128 * PSS + 2 * SLOT) * 2 +
+                      (size_t)(4 * 128 + 128 + 256 + 64 + 64 + 128 + 128 + (NORM ? 8 * 128 : 0)) * 4;
   const long long n_items = (long long)BH * a.NC * (a.DHHV / 512);
   if (n_items >= (1ll << 31)) return "stream_hv: too many work items";
   if ((size_t)a.S * (size_t)a.DHHV * 2 >= ((size_t)1 << 32)) return "stream_hv: one (batch, head) slab of an input exceeds 4 GiB";
@@ -566,18 +615,21 @@ const char* launch_stream_hv_t(const ParHvArgs& a, int BH, hipStream_t stream) {
   int G = (int)(n_items < cus ? n_items : cus);
   if (G >= 8) G -= G % 8;
   const int n_rounds = (int)((n_items + G - 1) / G);
-  if (hipFuncSetAttribute((const void*)stream_hv_kernel<IS_DV, F16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
-      hipSuccess)
+  if (hipFuncSetAttribute((const void*)stream_hv_kernel<IS_DV, F16, NORM>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)smem) != hipSuccess)
     return "stream_hv: cannot raise the dynamic LDS limit";
-  hipLaunchKernelGGL((stream_hv_kernel<IS_DV, F16>), dim3(G), dim3(768), smem, stream, a, (int)n_items, n_rounds);
+  hipLaunchKernelGGL((stream_hv_kernel<IS_DV, F16, NORM>), dim3(G), dim3(768), smem, stream, a, (int)n_items, n_rounds);
   return nullptr;
 }
 }  // namespace
 
 const char* launch_stream_hv(const ParHvArgs& a, int BH, bool is_dv, hipStream_t stream) {
-  if (!stream_hv_supported(a)) return "stream_hv: unsupported shape (needs DHQK = 256, DHHV % 512 == 0, S % 128 == 0, no head norm)";
+  if (!stream_hv_supported(a))
+    return "stream_hv: unsupported shape (needs DHQK = 256, DHHV % 512 == 0, S % 128 == 0; with a head norm DHHV = 512)";
   if (a.stride < 1 || a.stride > kMaxStateStride) return "stream_hv: state stride out of range";
   if (is_dv) return a.f16 ? launch_stream_hv_t<true, true>(a, BH, stream) : launch_stream_hv_t<true, false>(a, BH, stream);
+  if (a.head_norm != 0)
+    return a.f16 ? launch_stream_hv_t<false, true, true>(a, BH, stream) : launch_stream_hv_t<false, false, true>(a, BH, stream);
   return a.f16 ? launch_stream_hv_t<false, true>(a, BH, stream) : launch_stream_hv_t<false, false>(a, BH, stream);
 }
 
