@@ -116,6 +116,9 @@ __global__ __launch_bounds__(768) void stream_hv_kernel(ParHvArgs a, int n_items
     // register set to LDS, request slab L into the set: three slabs are on their way at any time.  The destination in LDS travels with the data: byte offset of
     // the thread's first piece | slab kind << 20 (0 fragment-order rows, 1 state fragments, 3 value rows) | gate-vector
     // flag << 22; the thread's other seven pieces lie a fixed distance apart.
+    // the loaders go first wherever a SIMD has a choice: their stores and requests after a barrier are what the next
+    // step of everybody waits for (measured: 2-4 % on this kernel; in the window dQ / dK kernel it costs 2 %)
+    __builtin_amdgcn_s_setprio(2);
     const int p = (wave_all - 8) * 64 + lane;  // 0 .. 255: every thread moves eight 16-byte pieces of every slab
     const char* const Xn_b = (const char*)(IS_DV ? a.K : a.Q);
     const char* const Xo_b = (const char*)(IS_DV ? a.Q : a.K);
