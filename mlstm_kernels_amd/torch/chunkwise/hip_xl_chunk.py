@@ -151,16 +151,17 @@ def _fw_launch(q, k, v, i, f, c0, n0, m0, eps, siging, normalize, want_last, kee
     return H, c_last, n_last, m_last, ws, norm_rstd
 
 
-def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
+def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging, f32_as_f16=False):
     dev = require_gpu(q, k, v, i, f)
     B, NH, S, DHQK = q.shape
     assert k.shape == (B, NH, S, DHQK), f"k has wrong shape {tuple(k.shape)}"
     assert v.shape[:3] == (B, NH, S), f"v has wrong shape {tuple(v.shape)}"
     assert i.shape == (B, NH, S) and f.shape == (B, NH, S), "i and f must have shape (B, NH, S)"
-    # operand format of the matrix kernels: float16 when q is float16, bfloat16 otherwise
-    kd = torch.float16 if q.dtype == torch.float16 else torch.bfloat16
+    # operand format of the matrix kernels: float16 when q is float16 (or float32 and the caller asked for float16
+    # operands), bfloat16 otherwise
+    kd = torch.float16 if (q.dtype == torch.float16 or (q.dtype == torch.float32 and f32_as_f16)) else torch.bfloat16
     for t in (q, k, v):
-        if t.dtype == torch.float32:
+        if t.dtype == torch.float32 and not f32_as_f16:
             _warn_rounding_once(t.dtype)
     qb, kb, vb = (t.to(kd).contiguous() for t in (q, k, v))
     gate_dt = i.dtype if (i.dtype == f.dtype and i.dtype in (torch.bfloat16, torch.float16)) else torch.float32
@@ -178,7 +179,7 @@ def _prep_inputs(q, k, v, i, f, c0, n0, m0, siging):
 
 
 def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, stride: int, norm: int, norm_eps: float,
-               recompute: bool):
+               recompute: bool, f32_as_f16: bool = False):
     class _HipChunkwiseFwBw(torch.autograd.Function):
         @staticmethod
         @custom_fwd(device_type="cuda", cast_inputs=autocast_kernel_dtype)
@@ -187,7 +188,7 @@ def _make_fwbw(autocast_kernel_dtype, siging: bool, normalize: bool, path: int, 
             # freshly allocated zero tensors the size of the state
             ctx.set_materialize_grads(False)
             out_dtype = q.dtype
-            dev, qb, kb, vb, ib, fb, c0f, n0f, m0f = _prep_inputs(q, k, v, i, f, c0, n0, m0, siging)
+            dev, qb, kb, vb, ib, fb, c0f, n0f, m0f = _prep_inputs(q, k, v, i, f, c0, n0, m0, siging, f32_as_f16)
             needs_bw = any(ctx.needs_input_grad[:6])
             H, c_last, n_last, m_last, ws, norm_rstd = _fw_launch(
                 qb, kb, vb, ib, fb, c0f, n0f, m0f, eps, siging, normalize, return_last_states, needs_bw, path, stride,
@@ -268,17 +269,23 @@ _FWBW_CACHE: dict = {}
 
 
 def _get_fwbw(autocast_kernel_dtype: torch.dtype, siging: bool, normalize: bool, kernel_path: str, stride: int,
-              head_norm: str = "none", head_norm_eps: float = 1e-6, recompute: bool = False):
+              head_norm: str = "none", head_norm_eps: float = 1e-6, recompute: bool = False,
+              float32_operands: str = "bfloat16"):
     if autocast_kernel_dtype not in (torch.float32, torch.float16, torch.bfloat16):
         raise ValueError(f"Unsupported kernel dtype {autocast_kernel_dtype}.")
     path = _lib.path_code(kernel_path)
     norm = _lib.norm_code(head_norm)
     if norm != _lib.NORM_NONE and path == _lib.PATH_FUSED:
         raise ValueError("head_norm is fused into the split kernel path only (kernel_path='auto' or 'split')")
-    key = (autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps), bool(recompute))
+    if float32_operands not in ("bfloat16", "float16"):
+        raise ValueError(f"float32_operands must be 'bfloat16' or 'float16', got {float32_operands!r}")
+    f32_as_f16 = float32_operands == "float16"
+    if f32_as_f16 and path == _lib.PATH_FUSED:
+        raise ValueError("the fused kernel path multiplies bfloat16 operands only")
+    key = (autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps), bool(recompute), f32_as_f16)
     if key not in _FWBW_CACHE:
         _FWBW_CACHE[key] = _make_fwbw(autocast_kernel_dtype, siging, normalize, path, stride, norm, float(head_norm_eps),
-                                      bool(recompute))
+                                      bool(recompute), f32_as_f16)
     return _FWBW_CACHE[key]
 
 
@@ -299,6 +306,7 @@ def mlstm_chunkwise__hip_xl_chunk(
     kernel_path: str = "auto",
     head_norm: str = "none",
     head_norm_eps: float = 1e-6,
+    float32_operands: str = "bfloat16",
     **tuning_kwargs,
 ):
     """mLSTMexp TFLA forward (+ autograd backward).  Returns ``H`` (dtype of q) or
@@ -310,6 +318,10 @@ def mlstm_chunkwise__hip_xl_chunk(
     (fwbw.py:222-241) -- means bfloat16 OPERANDS here: the matrix kernels multiply in the dtype of q, bfloat16 or
     float16, with fp32 accumulation, gates, normalisers and states; float32 inputs are rounded to bfloat16 with a
     one-time warning (about 1e-2 relative error in H against the float32 recurrence on the unrounded inputs).
+    ``float32_operands="float16"`` (not in the reference) rounds float32 inputs to float16 instead: the 11-bit
+    significand of the TF32 arithmetic the reference's float32 kernels run in on NVIDIA GPUs (about 1e-3 relative
+    error in H and the gradients), but float16's range -- values above 65504 overflow and gradients below 6e-8 vanish, which is why it
+    is not the default.
     ``chunk_size`` is validated like the reference does; 256 or more also sets the distance between kept states
     (as the reference's chunk_size_intra default does), 128 leaves it to the library.
     ``any_sequence_length=True`` (not in the reference) skips the reference's shape rules: the kernels mask a ragged
@@ -325,7 +337,7 @@ def mlstm_chunkwise__hip_xl_chunk(
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
     fn = _get_fwbw(autocast_kernel_dtype, False, True, kernel_path, stride, head_norm, head_norm_eps,
-                   _recompute_states(tuning_kwargs))
+                   _recompute_states(tuning_kwargs), float32_operands)
     H, c_last, n_last, m_last = fn.apply(q, k, v, i, f, c_initial, n_initial, m_initial, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last, m_last)
@@ -350,15 +362,17 @@ def mlstm_siging_chunkwise__hip_xl_chunk(
     kernel_path: str = "auto",
     head_norm: str = "none",
     head_norm_eps: float = 1e-6,
+    float32_operands: str = "bfloat16",
     **tuning_kwargs,
 ):
     """mLSTMsig (sigmoid input gate) TFLA forward (+ autograd backward).  Returns ``H`` or ``(H, (C_last, n_last))``.
-    ``any_sequence_length``, ``kernel_path``, ``chunk_size_intra`` and ``head_norm`` as for the exp gate."""
+    ``any_sequence_length``, ``kernel_path``, ``chunk_size_intra``, ``head_norm`` and ``float32_operands`` as for the
+    exp gate."""
     stride = _state_stride(tuning_kwargs, "mlstm_siging_chunkwise__hip_xl_chunk", chunk_size)
     if not any_sequence_length:
         validate_xl_chunk_shapes(q.shape[2], chunk_size)
     fn = _get_fwbw(autocast_kernel_dtype, True, bool(normalize), kernel_path, stride, head_norm, head_norm_eps,
-                   _recompute_states(tuning_kwargs))
+                   _recompute_states(tuning_kwargs), float32_operands)
     H, c_last, n_last, _ = fn.apply(q, k, v, i, f, c_initial, n_initial, None, return_last_states, eps)
     if return_last_states:
         return H, (c_last, n_last)

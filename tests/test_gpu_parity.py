@@ -499,6 +499,34 @@ def test_float32_inputs_run_with_bfloat16_operands():
     assert 5e-3 <= e <= 2e-2, f"norm error {e:.2e}: not the bfloat16 operand path's"
 
 
+def test_float32_inputs_with_float16_operands():
+    """float32_operands="float16": float32 inputs rounded to float16 (the 11-bit significand of the TF32 arithmetic the
+    reference's float32 Triton kernels use on NVIDIA GPUs) instead of bfloat16.  Full-mantissa float32 inputs, forward
+    and backward against the fp64 oracle on the UNROUNDED values: every element of H, dQ, dK, dV inside the plain
+    2e-2/2e-2 bound but at most one in 10^4, norm error below 3e-3 (measured 0.9e-3 .. 1.0e-3) -- a tenth of the
+    bfloat16 operand path's."""
+    exp_op, *_ = _ops()
+    if _VARIANT["kernel_path"] == "fused":
+        pytest.skip("the fused path multiplies bfloat16 operands only")
+    B, NH, S, DQK, DHV = 1, 2, 512, 256, 512
+    g = torch.Generator().manual_seed(321)
+    q, k, v, dH = (torch.randn(B, NH, S, d, generator=g) for d in (DQK, DQK, DHV, DHV))
+    i, f = torch.randn(B, NH, S, generator=g), 3 + torch.randn(B, NH, S, generator=g)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (q, k, v, i, f)]
+    H = exp_op(*leaves, chunk_size=128, autocast_kernel_dtype=torch.float32, float32_operands="float16")
+    assert H.dtype == torch.float32
+    H.backward(dH.to(DEV))
+    ref = O.chunkwise_fw(*(d64(t) for t in (q, k, v, i, f)), chunk_size=128)
+    bw = O.chunkwise_bw(*(d64(t) for t in (q, k, v, i, f)), d64(dH), chunk_size=128)
+    for name, x, r_ in [("H", H, ref["H"]), ("dQ", leaves[0].grad, bw[0]), ("dK", leaves[1].grad, bw[1]),
+                        ("dV", leaves[2].grad, bw[2])]:
+        assert x.dtype == torch.float32
+        check_matrix(x, r_, name, frac=1e-4, worst_tol=4.0, scale_tol=2e-3, norm_tol=3e-3)
+        print(f"    float16 operands, {name}: norm error {rel_norm(x, r_):.2e}")
+    with pytest.raises(ValueError, match="float32_operands"):
+        exp_op(*leaves, chunk_size=128, float32_operands="float64")
+
+
 def test_unsupported_head_dim_fails_loudly():
     exp_op, *_ = _ops()
     for dqk in (960, 1024):
