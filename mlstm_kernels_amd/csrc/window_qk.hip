@@ -360,10 +360,10 @@ __global__ __launch_bounds__(768) void window_qk_kernel(ParQkArgs a, int n_items
         for (int w = 0; w < NV; ++w) {
           __syncthreads();
           const unsigned char* const Cf = next_slab();
-          if (w == 0) {
-            finish_rowdots();
-            if (tid < 256) csv[tid] = csn;   // (read after the last step of this loop: NV - 1 >= 1 barriers later)
-          }
+          if (w == 0) finish_rowdots();
+          // (one step after the request, so that its latency hides behind the first step; read after the last step of
+          // this loop, at least one barrier later)
+          if (w == (NV > 2 ? 1 : 0) && tid < 256) csv[tid] = csn;
           const unsigned char* const Xn = Cf + 16384;
           const int le = opaque(lane);
           const int r = le & 31, h = le >> 5;
