@@ -311,3 +311,19 @@ def test_recurrent_sequence_rejects_what_it_does_not_implement():
         mlstm_recurrent_sequence__hip(t, t, t, g, g, return_all_states=True)
     with pytest.raises(TypeError, match="unexpected keyword"):
         mlstm_recurrent_sequence__hip(t, t, t, g, g, no_such_option=1)
+
+
+def test_float32_operand_option_is_validated_before_anything_runs():
+    """float32_operands: "bfloat16" (default) or "float16" for float32 inputs; anything else, or float16 on the fused
+    path (which multiplies bfloat16 operands only), is rejected when the operator is built."""
+    import pytest
+    import torch
+    from mlstm_kernels_amd.torch.chunkwise.hip_xl_chunk import _get_fwbw
+
+    a = _get_fwbw(torch.float32, False, True, "auto", 0)
+    b = _get_fwbw(torch.float32, False, True, "auto", 0, float32_operands="float16")
+    assert a is not b and a is _get_fwbw(torch.float32, False, True, "auto", 0, float32_operands="bfloat16")
+    with pytest.raises(ValueError, match="float32_operands"):
+        _get_fwbw(torch.float32, False, True, "auto", 0, float32_operands="float32")
+    with pytest.raises(ValueError, match="bfloat16 operands only"):
+        _get_fwbw(torch.float32, False, True, "fused", 0, float32_operands="float16")
